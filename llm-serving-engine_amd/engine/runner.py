@@ -187,8 +187,8 @@ class ModelRunner:
         self.cache_config = cache_config or CacheConfig()
         if max_sequence_length is None:
             max_sequence_length = getattr(loaded.config, "max_position_embeddings", None)
-        if max_sequence_length is None:
-            raise ValueError("max_sequence_length is needed for a config without max_position_embeddings")
+        if max_sequence_length is None:  # a model without a longest context: as long as the cache could hold
+            max_sequence_length = self.cache_config.num_blocks * self.cache_config.block_size
         tensors = {name: kernels.to_device(value) for name, value in loaded.tensors.items()}
         self.model = DecoderModel(loaded.spec, tensors, kernels)
         self.cache = CacheManager(

@@ -1,3 +1,3 @@
-from . import qwen2  # registers Qwen2ForCausalLM
+from . import dafutar, qwen2  # register Dafutar and Qwen2ForCausalLM
 
-__all__ = ["qwen2"]
+__all__ = ["dafutar", "qwen2"]

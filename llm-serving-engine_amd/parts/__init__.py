@@ -4,6 +4,7 @@ from .base import (
     LOGIT_PARTS,
     MIXERS,
     NORMS,
+    PASS_PARTS,
     POSITIONS,
     CacheNeed,
     FixedState,
@@ -15,11 +16,14 @@ from .base import (
     STREAM_PARTS,
     TensorSpec,
 )
-from .norm import RMSNorm, RMSNormSpec
-from .position import HeadLayout, NoPositionSpec, PositionEncoding, Rotary, RotarySpec
+from .norm import LayerNorm, LayerNormSpec, RMSNorm, RMSNormSpec
+from .position import HeadLayout, NoPositionSpec, PositionEncoding, Rotary, RotarySpec, YarnScaling, rotary_frequencies
 from .attention import Attention, AttentionSpec, Mixer
 from .feed_forward import FeedForward, GatedMLP, GatedMLPSpec
 from .block import Block, PreNormBlock, PreNormBlockSpec
-from .model import DecoderModel, LayerDefinition, LayerRun, ModelSpec, NamedPart
+from .model import DecoderModel, JoinedPass, JoinedPassSpec, LayerDefinition, LayerRun, ModelSpec, NamedPart
+from .latent_attention import LatentAttention, LatentAttentionSpec
+from .delta import GatedDelta, GatedDeltaSpec
+from .experts import RoutedExperts, RoutedExpertsSpec
 
 __all__ = [name for name in dir() if not name.startswith("_")]

@@ -193,6 +193,11 @@ BLOCKS = Registry("block")
 # `ModelSpec.output_parts`.
 STREAM_PARTS = Registry("part on the embedded stream")
 LOGIT_PARTS = Registry("part on the logits")
+# What stands at the start of a pass through a run of layers that a model walks several times: `forward(hidden,
+# delta, embedded, batch, number of the pass) -> hidden`, where `embedded` is the stream as it left the
+# embedding (and the input parts).  A model names one in `ModelSpec.pass_entry`, and the runs that begin a
+# pass in `LayerRun.enters`.
+PASS_PARTS = Registry("part at the start of a pass")
 
 
 def under(tensors: dict[str, Any], prefix: str) -> dict[str, Any]:

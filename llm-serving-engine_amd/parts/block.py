@@ -22,7 +22,8 @@ class Block(Part):
 @dataclass(frozen=True)
 class PreNormBlockSpec:
     """h += mixer(norm(h)); h += feed_forward(norm(h)).  The `*_name` fields are
-    the prefixes of the sub-parts' tensors below the layer's own prefix."""
+    the prefixes of the sub-parts' tensors below the layer's own prefix.  A layer without a
+    feed-forward has `feed_forward` None (and no norm for it)."""
 
     mixer_norm: Any
     mixer: Any
@@ -42,12 +43,11 @@ class PreNormBlock(Block):
 
     @classmethod
     def _members(cls, spec: PreNormBlockSpec):
-        return (
-            (spec.mixer_norm_name, NORMS, spec.mixer_norm),
-            (spec.mixer_name, MIXERS, spec.mixer),
-            (spec.feed_forward_norm_name, NORMS, spec.feed_forward_norm),
-            (spec.feed_forward_name, FEED_FORWARDS, spec.feed_forward),
-        )
+        members = [(spec.mixer_norm_name, NORMS, spec.mixer_norm), (spec.mixer_name, MIXERS, spec.mixer)]
+        if spec.feed_forward is not None:
+            members.append((spec.feed_forward_norm_name, NORMS, spec.feed_forward_norm))
+            members.append((spec.feed_forward_name, FEED_FORWARDS, spec.feed_forward))
+        return tuple(members)
 
     @classmethod
     def tensors(cls, spec: PreNormBlockSpec) -> dict[str, TensorSpec]:
@@ -66,11 +66,14 @@ class PreNormBlock(Block):
             registry.build(member, under(tensors, name), kernels)
             for name, registry, member in self._members(spec)
         ]
-        self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward = built
+        self.mixer_norm, self.mixer = built[:2]
+        self.feed_forward_norm, self.feed_forward = built[2:] if len(built) > 2 else (None, None)
         self.replayable = all(part.replayable for part in built)
 
     def forward(self, hidden, delta, batch, cell) -> torch.Tensor:
         normed = self.mixer_norm.forward(hidden, delta)
         mixed = self.mixer.forward(normed, batch, cell)
+        if self.feed_forward is None:
+            return mixed
         normed = self.feed_forward_norm.forward(hidden, mixed)
         return self.feed_forward.forward(normed, batch)

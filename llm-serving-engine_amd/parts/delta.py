@@ -1,0 +1,94 @@
+"""A recurrent mixer: the gated delta rule over a matrix state per head, behind short causal convolutions."""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from .attention import Mixer
+from .base import MIXERS, FixedState, TensorSpec
+
+
+@dataclass(frozen=True)
+class GatedDeltaSpec:
+    """`num_heads` value heads of `vdim`, `num_kv_heads` query/key heads of `dim` (value head h reads
+    query/key head h // (num_heads / num_kv_heads)); `taps` of the convolutions; `eps` of the output norm."""
+
+    hidden_size: int
+    num_heads: int
+    num_kv_heads: int
+    dim: int
+    vdim: int
+    taps: int
+    eps: float
+    kind: str = "gated_delta"
+
+    @property
+    def channels(self) -> int:
+        """q, k and v side by side: what the convolutions run over."""
+        return 2 * self.num_kv_heads * self.dim + self.num_heads * self.vdim
+
+
+@MIXERS.register("gated_delta")
+class GatedDelta(Mixer):
+    """q, k, v = silu(conv(W x)) per channel over the last `taps` tokens; q and k made unit vectors per head
+    (x / sqrt(sum x^2 + 1e-6)), q times dim^-1/2; per value head beta = sigmoid(W_b x) and the decay
+    g = exp(-exp(A_log) softplus(W_a x + dt_bias)).  Token by token, per head, with S [dim, vdim]:
+
+        S = g S;   u = beta (v - S^T k);   S = S + k u^T;   o = S^T q
+
+    then o / rms(o) * norm * silu(W_g x) head by head, and W_o.  Decay, beta, the unit norms and S are
+    float32.  Per request the cache keeps S and the last `taps - 1` inputs of the convolutions, both in
+    state slots that are zero when a request begins."""
+
+    @classmethod
+    def tensors(cls, spec: GatedDeltaSpec) -> dict[str, TensorSpec]:
+        qk, v = spec.num_kv_heads * spec.dim, spec.num_heads * spec.vdim
+        return {
+            "q": TensorSpec((qk, spec.hidden_size)),
+            "q.conv": TensorSpec((qk, spec.taps)),
+            "k": TensorSpec((qk, spec.hidden_size)),
+            "k.conv": TensorSpec((qk, spec.taps)),
+            "v": TensorSpec((v, spec.hidden_size)),
+            "v.conv": TensorSpec((v, spec.taps)),
+            "b": TensorSpec((spec.num_heads, spec.hidden_size)),
+            "a": TensorSpec((spec.num_heads, spec.hidden_size)),
+            "A_log": TensorSpec((spec.num_heads,), role="bias"),
+            "dt_bias": TensorSpec((spec.num_heads,), role="bias"),
+            "norm": TensorSpec((spec.vdim,), role="norm"),
+            "g": TensorSpec((v, spec.hidden_size)),
+            "o": TensorSpec((spec.hidden_size, v)),
+        }
+
+    @classmethod
+    def cache_need(cls, spec: GatedDeltaSpec) -> dict[str, FixedState]:
+        need = {"state": FixedState((spec.num_heads, spec.dim, spec.vdim))}
+        if spec.taps > 1:
+            need["window"] = FixedState((spec.taps - 1, spec.channels))
+        return need
+
+    def __init__(self, spec: GatedDeltaSpec, tensors, kernels) -> None:
+        super().__init__(spec, tensors, kernels)
+        if spec.num_heads % spec.num_kv_heads:
+            raise ValueError("gated delta: the value heads are a multiple of the query/key heads")
+        # one product for what the convolutions and the output gate read, one (kept float32) for what enters the recurrence
+        self.inputs = kernels.prepare_linear([tensors[name] for name in ("q", "k", "v", "g")], None)
+        self.controls = kernels.prepare_linear([tensors["b"], tensors["a"]], None)
+        self.taps = kernels.to_device(torch.cat([tensors[name + ".conv"] for name in ("q", "k", "v")], dim=0).float().contiguous())
+        self.rate = kernels.to_device(tensors["A_log"].float().contiguous())
+        self.step_bias = kernels.to_device(tensors["dt_bias"].float().contiguous())
+        self.norm = tensors["norm"]
+        self.out = kernels.prepare_linear([tensors["o"]], None)
+
+    def forward(self, x: torch.Tensor, batch, cell) -> torch.Tensor:
+        kernels, spec = self.kernels, self.spec
+        projected = kernels.linear(x, self.inputs)  # [T, q | k | v | g]
+        controls = kernels.linear(x, self.controls, out_dtype=torch.float32)  # [T, b | a]
+        window = cell["window"].state if "window" in cell else None
+        mixed = kernels.causal_conv(projected, spec.channels, self.taps, "silu", batch, window)  # [T, q | k | v]
+        read = kernels.gated_delta_rule(
+            mixed, controls, self.rate, self.step_bias, spec.num_heads, spec.num_kv_heads, spec.dim, spec.vdim, batch, cell["state"].state
+        )  # float32 [T, heads * vdim]
+        gated = kernels.gated_head_norm(read, projected, spec.channels, self.norm, spec.eps, spec.num_heads, spec.vdim, "silu")
+        return kernels.linear(gated, self.out, out_dtype=torch.float32, partial=True)

@@ -24,6 +24,8 @@ class GatedMLPSpec:
     intermediate_size: int
     activation: str = "silu"
     kind: str = "gated_mlp"
+    # the tensors' names below the part's prefix: gate, up, down
+    names: tuple[str, str, str] = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")
 
 
 @FEED_FORWARDS.register("gated_mlp")
@@ -33,19 +35,19 @@ class GatedMLP(FeedForward):
 
     @classmethod
     def tensors(cls, spec: GatedMLPSpec) -> dict[str, TensorSpec]:
+        gate, up, down = spec.names
         return {
-            "gate_proj.weight": TensorSpec((spec.intermediate_size, spec.hidden_size)),
-            "up_proj.weight": TensorSpec((spec.intermediate_size, spec.hidden_size)),
-            "down_proj.weight": TensorSpec((spec.hidden_size, spec.intermediate_size)),
+            gate: TensorSpec((spec.intermediate_size, spec.hidden_size)),
+            up: TensorSpec((spec.intermediate_size, spec.hidden_size)),
+            down: TensorSpec((spec.hidden_size, spec.intermediate_size)),
         }
 
     def __init__(self, spec: GatedMLPSpec, tensors, kernels) -> None:
         super().__init__(spec, tensors, kernels)
         # the kernel library says which activations it has, and refuses another by name
-        self.gate_up = kernels.prepare_gated_linear(
-            tensors["gate_proj.weight"], tensors["up_proj.weight"], spec.activation
-        )
-        self.down = kernels.prepare_linear([tensors["down_proj.weight"]], None)
+        gate, up, down = spec.names
+        self.gate_up = kernels.prepare_gated_linear(tensors[gate], tensors[up], spec.activation)
+        self.down = kernels.prepare_linear([tensors[down]], None)
 
     def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
         activated = self.kernels.gated_linear(x, self.gate_up)

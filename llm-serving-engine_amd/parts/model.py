@@ -8,7 +8,7 @@ from typing import Any
 
 import torch
 
-from .base import BLOCKS, LOGIT_PARTS, NORMS, STREAM_PARTS, CacheNeed, TensorSpec, prefixed, under
+from .base import BLOCKS, LOGIT_PARTS, NORMS, PASS_PARTS, STREAM_PARTS, CacheNeed, TensorSpec, prefixed, under
 
 
 @dataclass(frozen=True)
@@ -22,10 +22,13 @@ class LayerRun:
     """One entry of the run order.  `layer` indexes `ModelSpec.layers`; a layer
     may be named by several entries (its tensors are shared, each run has a
     cache cell of its own).  With `reads` set, the run uses the cell of that
-    earlier entry of the run order instead, and stores nothing."""
+    earlier entry of the run order instead, and stores nothing.  With `enters` set, the run is
+    the first of a pass (its number: 0, 1, ...) through layers that the model walks several times, and
+    the model's `pass_entry` part acts on the stream before it."""
 
     layer: int
     reads: int | None = None
+    enters: int | None = None
 
 
 @dataclass(frozen=True)
@@ -51,8 +54,14 @@ class ModelSpec:
     # logits after the head (kinds of LOGIT_PARTS), in order; Qwen2 has none
     input_parts: tuple[NamedPart, ...] = ()
     output_parts: tuple[NamedPart, ...] = ()
+    # the part that stands before every run with `enters` set (a kind of PASS_PARTS)
+    pass_entry: NamedPart | None = None
+    # tensors that a model folder may hold and the model does not use
+    ignored_tensors: tuple[str, ...] = ()
 
     def __post_init__(self) -> None:
+        if self.pass_entry is None and any(run.enters is not None for run in self.run_order):
+            raise ValueError("a run begins a pass, and the model has no part for that")
         for index, run in enumerate(self.run_order):
             if not 0 <= run.layer < len(self.layers):
                 raise ValueError(f"run {index} names layer {run.layer}, which does not exist")
@@ -78,6 +87,8 @@ class ModelSpec:
             found.update(prefixed(STREAM_PARTS.tensors(part.spec), part.prefix))
         for part in self.output_parts:
             found.update(prefixed(LOGIT_PARTS.tensors(part.spec), part.prefix))
+        if self.pass_entry is not None:
+            found.update(prefixed(PASS_PARTS.tensors(self.pass_entry.spec), self.pass_entry.prefix))
         if not self.tie_embeddings:
             found[self.head_name] = TensorSpec((self.vocab_size, self.hidden_size))
         return found
@@ -100,16 +111,29 @@ class DecoderModel:
         self.head = kernels.prepare_linear([head], None)
         self.input_parts = [STREAM_PARTS.build(part.spec, under(tensors, part.prefix), kernels) for part in spec.input_parts]
         self.output_parts = [LOGIT_PARTS.build(part.spec, under(tensors, part.prefix), kernels) for part in spec.output_parts]
+        self.pass_entry = None
+        if spec.pass_entry is not None:
+            self.pass_entry = PASS_PARTS.build(spec.pass_entry.spec, under(tensors, spec.pass_entry.prefix), kernels)
         every = [*self.layers, self.final_norm, *self.input_parts, *self.output_parts]
+        every += [self.pass_entry] if self.pass_entry is not None else []
         self.replayable = all(part.replayable for part in every)
+        # Called, if set, after every run of the run order with (index of the run, the float32 stream, what the
+        # run still has to add to it: None, [T, hidden] or partial sums [parts, T, hidden]): tests and
+        # debugging look at the stream layer by layer through it (with a runner that replays no graphs).
+        self.observer = None
 
     def _run_layers(self, batch, cells: list):
         hidden = self.kernels.embedding(self.embedding, batch.token_ids)
         for part in self.input_parts:
             part.forward(hidden, batch)
+        embedded = hidden.clone() if self.pass_entry is not None else None  # the layers add into `hidden` in place
         delta = None
-        for run, cell in zip(self.spec.run_order, cells):
+        for index, (run, cell) in enumerate(zip(self.spec.run_order, cells)):
+            if run.enters is not None:
+                hidden, delta = self.pass_entry.forward(hidden, delta, embedded, batch, run.enters), None
             delta = self.layers[run.layer].forward(hidden, delta, batch, cell)
+            if self.observer is not None:
+                self.observer(index, hidden, delta)
         return hidden, delta
 
     def forward_without_logits(self, batch, cells: list) -> None:
@@ -129,3 +153,45 @@ class DecoderModel:
         for part in self.output_parts:
             logits = part.forward(logits, batch)
         return logits
+
+
+@dataclass(frozen=True)
+class JoinedPassSpec:
+    """x <- W [x; x0] + step[t] at the start of pass t, x0 the embedded stream; `passes` is how many
+    there are.  `weight_name` [hidden, 2 hidden] and `step_name` [passes, hidden] below the part's prefix."""
+
+    hidden_size: int
+    passes: int
+    weight_name: str = "in"
+    step_name: str = "step"
+    kind: str = "joined_pass"
+
+
+@PASS_PARTS.register("joined_pass")
+class JoinedPass:
+    """The stream that enters a pass is a product of the stream so far beside the embedded one, plus a
+    vector of the pass.  The product's operand is the two streams side by side in the run dtype; its result
+    (with the pass's vector as the product's bias) is the new float32 stream."""
+
+    replayable = True
+
+    @classmethod
+    def tensors(cls, spec: JoinedPassSpec) -> dict[str, TensorSpec]:
+        return {
+            spec.weight_name: TensorSpec((spec.hidden_size, 2 * spec.hidden_size)),
+            spec.step_name: TensorSpec((spec.passes, spec.hidden_size), role="bias"),
+        }
+
+    @classmethod
+    def cache_need(cls, spec: JoinedPassSpec) -> None:
+        return None
+
+    def __init__(self, spec: JoinedPassSpec, tensors, kernels) -> None:
+        self.spec = spec
+        self.kernels = kernels
+        weight, steps = tensors[spec.weight_name], tensors[spec.step_name]
+        self.products = [kernels.prepare_linear([weight], [steps[index].contiguous()]) for index in range(spec.passes)]
+
+    def forward(self, hidden, delta, embedded, batch, number: int):
+        both = self.kernels.join_rows(hidden, delta, embedded)  # [T, 2 hidden] in the run dtype
+        return self.kernels.linear(both, self.products[number], out_dtype=torch.float32)

@@ -33,3 +33,34 @@ class RMSNorm(Part):
     def forward(self, hidden: torch.Tensor, delta: torch.Tensor | None) -> torch.Tensor:
         """Adds `delta` into `hidden` (in place) and returns the normed rows in the run dtype."""
         return self.kernels.add_rms_norm(hidden, delta, self.weight, self.spec.eps)
+
+
+@dataclass(frozen=True)
+class LayerNormSpec:
+    """`weight_name` and `bias_name` are the tensors' names below the part's prefix (a model whose files
+    call them otherwise says so here)."""
+
+    size: int
+    eps: float
+    weight_name: str = "weight"
+    bias_name: str = "bias"
+    kind: str = "layernorm"
+
+
+@NORMS.register("layernorm")
+class LayerNorm(Part):
+    """y = (x - mean(x)) * rsqrt(mean((x - mean(x))^2) + eps) * weight + bias, all in float32, with the
+    residual add in front of it as in `RMSNorm`."""
+
+    @classmethod
+    def tensors(cls, spec: LayerNormSpec) -> dict[str, TensorSpec]:
+        return {spec.weight_name: TensorSpec((spec.size,), role="norm"), spec.bias_name: TensorSpec((spec.size,), role="bias")}
+
+    def __init__(self, spec: LayerNormSpec, tensors, kernels) -> None:
+        super().__init__(spec, tensors, kernels)
+        self.weight = tensors[spec.weight_name]
+        self.bias = tensors[spec.bias_name]
+
+    def forward(self, hidden: torch.Tensor, delta: torch.Tensor | None) -> torch.Tensor:
+        """Adds `delta` into `hidden` (in place) and returns the normed rows in the run dtype."""
+        return self.kernels.add_layer_norm(hidden, delta, self.weight, self.bias, self.spec.eps)

@@ -2,6 +2,7 @@
 
 from __future__ import annotations
 
+import math
 from dataclasses import dataclass
 
 import torch
@@ -92,3 +93,33 @@ class NoPosition(PositionEncoding):
 
     def encode_store_attend(self, qkv, layout: HeadLayout, batch, cell, scale: float, window, project=None):
         return self.kernels.rotate_store_attend(qkv, layout, batch, cell, None, "none", scale, window, project=project)
+
+
+@dataclass(frozen=True)
+class YarnScaling:
+    """Frequencies stretched for contexts longer than the `original` one: a pair whose wavelength makes more
+    than `fast` turns over the original context keeps its frequency, one that makes fewer than `slow` has it
+    divided by `factor`, a linear ramp over the pair index between; cosines and sines grow by 0.1 ln(factor) + 1."""
+
+    factor: float
+    original: float
+    fast: float
+    slow: float
+
+
+def rotary_frequencies(dims: int, theta: float, scaling: YarnScaling | None = None) -> tuple[torch.Tensor, float]:
+    """(float32 frequencies [dims / 2] of pair i, theta^(-2i / dims), stretched by `scaling`; what the cosines
+    and sines are multiplied by).  Computed in float64 and rounded once."""
+    index = torch.arange(dims // 2, dtype=torch.float64)
+    plain = float(theta) ** (-2.0 * index / dims)
+    if scaling is None:
+        return plain.to(torch.float32), 1.0
+
+    def turning_pair(turns: float) -> float:  # the (fractional) dimension whose wavelength makes `turns` turns over the original context
+        return dims * math.log(scaling.original / (2.0 * math.pi * turns)) / (2.0 * math.log(theta))
+
+    low = max(math.floor(turning_pair(scaling.fast)), 0)
+    high = min(math.ceil(turning_pair(scaling.slow)), dims - 1)
+    ramp = ((index - low) / max(high - low, 0.001)).clamp(0.0, 1.0)
+    stretched = plain / scaling.factor * ramp + plain * (1.0 - ramp)
+    return stretched.to(torch.float32), 0.1 * math.log(scaling.factor) + 1.0

@@ -47,8 +47,11 @@ def unregister_architecture(name: str) -> None:
 
 
 def resolve_architecture(config_values: dict[str, Any]) -> Architecture:
-    """Chooses by config.json's `architectures`, else by its `model_type`."""
-    for name in config_values.get("architectures") or ():
+    """Chooses by config.json's `architectures` (or its one `architecture`), else by its `model_type`."""
+    named = list(config_values.get("architectures") or ())
+    if isinstance(config_values.get("architecture"), str):
+        named.append(config_values["architecture"])
+    for name in named:
         if name in ARCHITECTURES:
             return ARCHITECTURES[name]
     model_type = config_values.get("model_type")
@@ -56,6 +59,6 @@ def resolve_architecture(config_values: dict[str, Any]) -> Architecture:
         if model_type is not None and model_type in entry.model_types:
             return entry
     raise ConfigError(
-        f"no registered architecture for architectures={config_values.get('architectures')!r}, "
+        f"no registered architecture for architectures={named!r}, "
         f"model_type={model_type!r} (registered: {sorted(ARCHITECTURES)})"
     )

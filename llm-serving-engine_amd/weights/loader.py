@@ -156,6 +156,8 @@ def load_model_folder(
             embedding, found[spec.head_name]
         ):
             del found[spec.head_name]
+    for name in spec.ignored_tensors:  # what the folder may hold and the model does not use
+        found.pop(name, None)
     fit_tensors(expected, found, str(folder))
     tensors = {
         name: _kept_as(found[name], expected[name], dtype).to(device).contiguous() for name in expected

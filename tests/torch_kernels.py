@@ -148,3 +148,139 @@ class TorchKernels:
             hit = torch.nonzero(running > u * running[-1])
             chosen.append(int(order[hit[0, 0]] if hit.numel() else order[-1]))
         return torch.tensor(chosen, dtype=torch.int32)
+
+    # ------------------------------------------------------------------ layer norm, column-wise operations
+
+    def add_layer_norm(self, hidden, delta, weight, bias, eps):
+        if delta is not None:
+            hidden += delta if delta.ndim == 2 else delta.sum(0)
+        mean = hidden.mean(-1, keepdim=True)
+        centred = hidden - mean
+        variance = centred.pow(2).mean(-1, keepdim=True)
+        return (centred * torch.rsqrt(variance + eps) * weight.float() + bias.float()).to(self.dtype)
+
+    def new_rows(self, rows, width):
+        return torch.zeros((rows, width), dtype=self.dtype)
+
+    def rms_norm_columns(self, x, first, weight, eps, out=None, out_first=0, copies=1, copy_stride=0):
+        width = weight.shape[0]
+        part = x[:, first : first + width].float()
+        normed = (part * torch.rsqrt(part.pow(2).mean(-1, keepdim=True) + eps) * weight.float()).to(self.dtype)
+        if out is None:
+            return normed
+        for copy in range(copies):
+            out[:, out_first + copy * copy_stride : out_first + copy * copy_stride + width] = normed
+        return out
+
+    def rotary_table(self, batch, frequencies, magnitude=1.0):
+        angles = batch.positions.float()[:, None] * frequencies.float()[None, :]
+        return torch.stack([angles.cos() * magnitude, angles.sin() * magnitude], dim=-1)
+
+    def rotate_columns(self, x, first, head_stride, heads, width, table, dims, out, out_first, out_head_stride):
+        cos, sin = table[..., 0], table[..., 1]
+        for head in range(heads):
+            part = x[:, first + head * head_stride : first + head * head_stride + width].float()
+            turned = part.clone()
+            a, b = part[:, 0:dims:2], part[:, 1:dims:2]
+            turned[:, 0:dims:2] = a * cos - b * sin
+            turned[:, 1:dims:2] = b * cos + a * sin
+            out[:, out_first + head * out_head_stride : out_first + head * out_head_stride + width] = turned.to(out.dtype)
+        return out
+
+    def prepare_headwise_linear(self, weight):
+        return weight.float()
+
+    def headwise_linear(self, x, first, head_stride, weights, out=None, out_first=0, out_head_stride=None):
+        heads, outputs, inner = weights.shape
+        stride = outputs if out_head_stride is None else out_head_stride
+        if out is None:
+            out = torch.zeros((x.shape[0], heads * outputs), dtype=self.dtype)
+        for head in range(heads):
+            part = x[:, first + head * head_stride : first + head * head_stride + inner].float()
+            out[:, out_first + head * stride : out_first + head * stride + outputs] = (part @ weights[head].T).to(out.dtype)
+        return out
+
+    def join_rows(self, hidden, delta, embedded):
+        now = hidden if delta is None else hidden + (delta if delta.ndim == 2 else delta.sum(0))
+        return torch.cat([now, embedded], dim=-1).to(self.dtype)
+
+    def activate(self, x, activation):
+        acts = {"silu": torch.nn.functional.silu, "gelu": torch.nn.functional.gelu, "relu": torch.relu,
+                "gelu_tanh": lambda z: torch.nn.functional.gelu(z, approximate="tanh")}
+        return acts[activation](x.float()).to(x.dtype)
+
+    def add_gated_rows(self, target, rows, gates, column, squash):
+        assert squash == "sigmoid"
+        target += torch.sigmoid(gates[:, column : column + 1].float()) * rows
+        return target
+
+    # ------------------------------------------------------------------ the gated delta rule
+
+    def causal_conv(self, x, channels, taps, activation, batch, window):
+        assert activation == "silu"
+        width = taps.shape[1]
+        out = torch.zeros((x.shape[0], channels))
+        row = 0
+        for chunk in batch.chunks:
+            fresh = x[row : row + chunk.count, :channels].float()
+            before = window[chunk.slot] if window is not None else torch.zeros((0, channels))
+            line = torch.cat([before, fresh])  # the last taps - 1 inputs, then this step's
+            for j in range(width):
+                out[row : row + chunk.count] += line[j : j + chunk.count] * taps[:, j]
+            if window is not None:
+                window[chunk.slot] = line[-(width - 1):]
+            row += chunk.count
+        return torch.nn.functional.silu(out).to(self.dtype)
+
+    def gated_delta_rule(self, mixed, controls, rate, step_bias, heads, kv_heads, dim, vdim, batch, state):
+        tokens = mixed.shape[0]
+        q = mixed[:, : kv_heads * dim].float().view(tokens, kv_heads, dim)
+        k = mixed[:, kv_heads * dim : 2 * kv_heads * dim].float().view(tokens, kv_heads, dim)
+        v = mixed[:, 2 * kv_heads * dim :].float().view(tokens, heads, vdim)
+        q = q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + 1e-6) * dim**-0.5
+        k = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)
+        beta = torch.sigmoid(controls[:, :heads].float())
+        decay = torch.exp(-torch.exp(rate.float()) * torch.nn.functional.softplus(controls[:, heads:].float() + step_bias.float()))
+        out = torch.zeros((tokens, heads, vdim))
+        row = 0
+        for chunk in batch.chunks:
+            S = state[chunk.slot]  # [heads, dim, vdim], updated in place
+            for t in range(row, row + chunk.count):
+                kt = k[t].repeat_interleave(heads // kv_heads, dim=0)
+                qt = q[t].repeat_interleave(heads // kv_heads, dim=0)
+                S *= decay[t].view(heads, 1, 1)
+                u = beta[t].view(heads, 1) * (v[t] - torch.einsum("hdv,hd->hv", S, kt))
+                S += torch.einsum("hd,hv->hdv", kt, u)
+                out[t] = torch.einsum("hdv,hd->hv", S, qt)
+            row += chunk.count
+        return out.reshape(tokens, heads * vdim)
+
+    def gated_head_norm(self, read, gates, gate_first, weight, eps, heads, vdim, activation):
+        assert activation == "silu"
+        tokens = read.shape[0]
+        rows = read.view(tokens, heads, vdim)
+        normed = rows * torch.rsqrt(rows.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+        gate = torch.nn.functional.silu(gates[:, gate_first : gate_first + heads * vdim].float()).view(tokens, heads, vdim)
+        return (normed * gate).reshape(tokens, heads * vdim).to(self.dtype)
+
+    # ------------------------------------------------------------------ routed experts
+
+    def route(self, scores, experts, correction, top, scale, scoring):
+        assert scoring == "sigmoid"
+        squashed = torch.sigmoid(scores[:, :experts].float())
+        choice = squashed + correction.float()
+        chosen = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :top]
+        return chosen.to(torch.int32), (squashed.gather(1, chosen) * scale).float()
+
+    def prepare_experts(self, ups, downs, activation):
+        return (torch.stack([w.float() for w in ups]), torch.stack([w.float() for w in downs]), activation)
+
+    def expert_feed_forward(self, x, experts, chosen, weights):
+        ups, downs, activation = experts
+        out = torch.zeros((x.shape[0], downs.shape[1]))
+        for t in range(x.shape[0]):
+            for slot in range(chosen.shape[1]):
+                e = int(chosen[t, slot])
+                inner = self.activate((x[t].float() @ ups[e].T).to(self.dtype), activation).float()
+                out[t] += weights[t, slot] * (inner @ downs[e].T)
+        return out
