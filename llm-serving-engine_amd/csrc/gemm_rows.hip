@@ -1,0 +1,256 @@
+// Products whose rows or weights are chosen per tile: a product per head over a run of a row's columns, and the
+// products of routed experts over rows that were sorted by expert on the device.  One core: a workgroup of 256
+// threads makes a 16 x 64 tile of the result, K in steps of 32 through LDS, float32 arithmetic and sums in the
+// order of k whatever the batch holds.  Operands are bfloat16 or float32.
+#include "common.h"
+
+#define TILE_ROWS 16
+#define TILE_COLS 64
+#define TILE_K 32
+#define PAD_K 33
+
+#define ACT_NONE -1
+#define ACT_SILU 0
+#define ACT_GELU 1
+#define ACT_GELU_TANH 2
+#define ACT_RELU 3
+
+__device__ __forceinline__ float activation_of(int activation, float z) {
+  switch (activation) {
+    case ACT_NONE: return z;
+    case ACT_GELU: return 0.5f * z * (1.f + erff(z * 0.70710678118654752f));
+    case ACT_GELU_TANH: return 0.5f * z * (1.f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
+    case ACT_RELU: return fmaxf(z, 0.f);
+    default: return z / (1.f + expf(-z));
+  }
+}
+
+// Thread t loads two elements of x row t / 16 and eight of weight row t / 4 per step, and owns the results
+// (row t / 16, columns t % 16 + 16 j).  `x_row` / `w_row` are the thread's rows to load (null: zeros).
+template <typename TX, typename TW>
+__device__ __forceinline__ void tile_product(const TX* x_row, const TW* w_row, int inner, float (&acc)[4], float* xs, float* ws) {
+  const int t = threadIdx.x, r = t / 16, g = t % 16;
+  const int xk = (t % 16) * 2, wn = t / 4, wk = (t % 4) * 8;
+  for (int k0 = 0; k0 < inner; k0 += TILE_K) {
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int k = k0 + xk + e;
+      xs[r * PAD_K + xk + e] = (x_row && k < inner) ? to_float(x_row[k]) : 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int k = k0 + wk + e;
+      ws[wn * PAD_K + wk + e] = (w_row && k < inner) ? to_float(w_row[k]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < TILE_K; ++kk) {
+      const float a = xs[r * PAD_K + kk];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] += a * ws[(g + 16 * j) * PAD_K + kk];
+    }
+    __syncthreads();
+  }
+}
+
+// ---------------------------------------------------------------------------- a product per head
+// out[t, out_first + h * out_head_stride + n] = sum_k x[t, first + h * head_stride + k] * w[h, n, k]
+template <typename T>
+__global__ __launch_bounds__(256) void headwise_kernel(const T* __restrict__ x, int x_stride, int first, int head_stride,
+                                                       const T* __restrict__ w, int outputs, int inner, T* __restrict__ out,
+                                                       int out_stride, int out_first, int out_head_stride, int rows) {
+  __shared__ float xs[TILE_ROWS * PAD_K], ws[TILE_COLS * PAD_K];
+  const int head = blockIdx.z, row0 = blockIdx.y * TILE_ROWS, col0 = blockIdx.x * TILE_COLS;
+  const int t = threadIdx.x;
+  const int load_row = row0 + t / 16, load_col = col0 + t / 4;
+  const T* x_row = load_row < rows ? x + (size_t)load_row * x_stride + first + (size_t)head * head_stride : nullptr;
+  const T* w_row = load_col < outputs ? w + ((size_t)head * outputs + load_col) * inner : nullptr;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  tile_product(x_row, w_row, inner, acc, xs, ws);
+  const int row = row0 + t / 16;
+  if (row >= rows) return;
+  T* dst = out + (size_t)row * out_stride + out_first + (size_t)head * out_head_stride;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int n = col0 + t % 16 + 16 * j;
+    if (n < outputs) dst[n] = from_float<T>(acc[j]);
+  }
+}
+
+extern "C" int llmserve_headwise_linear(const void* x, int is_float, int rows, int x_stride, int first, int head_stride,
+                                        const void* w, int heads, int outputs, int inner, void* out, int out_stride,
+                                        int out_first, int out_head_stride, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (heads < 1 || outputs < 1 || inner < 1 || first + (heads - 1) * head_stride + inner > x_stride ||
+      out_first + (heads - 1) * out_head_stride + outputs > out_stride || heads > 65535)
+    return ERR_BAD_ARGUMENT;
+  const dim3 grid((outputs + TILE_COLS - 1) / TILE_COLS, (rows + TILE_ROWS - 1) / TILE_ROWS, heads);
+  if (grid.y > 65535) return ERR_BAD_ARGUMENT;
+  if (is_float)
+    hipLaunchKernelGGL(headwise_kernel<float>, grid, dim3(256), 0, stream, (const float*)x, x_stride, first, head_stride,
+                       (const float*)w, outputs, inner, (float*)out, out_stride, out_first, out_head_stride, rows);
+  else
+    hipLaunchKernelGGL(headwise_kernel<bf16_t>, grid, dim3(256), 0, stream, (const bf16_t*)x, x_stride, first, head_stride,
+                       (const bf16_t*)w, outputs, inner, (bf16_t*)out, out_stride, out_first, out_head_stride, rows);
+  return LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------- routing
+// One thread a token: s_e = sigmoid(z[t, e]); the `top` experts with the largest s_e + correction_e, the lower index
+// first among equals; chosen[t, i] and weight[t, i] = scale * s_e (no renormalising).
+__global__ void route_kernel(const float* __restrict__ z, int z_stride, int experts, const float* __restrict__ correction,
+                             int top, float scale, int* __restrict__ chosen, float* __restrict__ weight, int tokens) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= tokens) return;
+  const float* row = z + (size_t)t * z_stride;
+  int* mine = chosen + (size_t)t * top;
+  for (int i = 0; i < top; ++i) {
+    int best = -1;
+    float best_choice = 0.f, best_score = 0.f;
+    for (int e = 0; e < experts; ++e) {
+      bool taken = false;
+      for (int j = 0; j < i; ++j) taken |= mine[j] == e;
+      if (taken) continue;
+      const float score = 1.f / (1.f + expf(-row[e]));
+      const float choice = score + correction[e];
+      if (best < 0 || choice > best_choice) { best = e; best_choice = choice; best_score = score; }
+    }
+    mine[i] = best;
+    weight[(size_t)t * top + i] = scale * best_score;
+  }
+}
+
+extern "C" int llmserve_route(const float* z, int z_stride, int experts, const float* correction, int top, float scale,
+                              int* chosen, float* weight, int tokens, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (experts < 1 || top < 1 || top > experts || experts > z_stride) return ERR_BAD_ARGUMENT;
+  hipLaunchKernelGGL(route_kernel, dim3((tokens + 127) / 128), dim3(128), 0, stream, z, z_stride, experts, correction, top,
+                     scale, chosen, weight, tokens);
+  return LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------- sorting the (token, choice) pairs by expert
+// One workgroup.  place[p] is where pair p = t * top + i stands in the order by expert (the order within an expert is
+// whichever the counting gave: every row is computed by itself, so results do not depend on it); order[place[p]] = p.
+// The tiles of the grouped products, TILE_ROWS rows of one expert each: tile[i] = (expert, first place, rows); there is
+// room for ceil(pairs / TILE_ROWS) + experts of them, and those not needed have no rows.
+#define SORT_THREADS 1024
+#define MAX_EXPERTS 1024
+__global__ __launch_bounds__(SORT_THREADS) void sort_pairs_kernel(const int* __restrict__ chosen, int pairs, int experts,
+                                                                  int* __restrict__ place, int* __restrict__ order,
+                                                                  int* __restrict__ tiles, int capacity) {
+  __shared__ int count[MAX_EXPERTS], first[MAX_EXPERTS], first_tile[MAX_EXPERTS + 1];
+  for (int e = threadIdx.x; e < experts; e += SORT_THREADS) count[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += SORT_THREADS) place[p] = atomicAdd(&count[chosen[p]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int rows = 0, tile = 0;
+    for (int e = 0; e < experts; ++e) {
+      first[e] = rows;
+      first_tile[e] = tile;
+      rows += count[e];
+      tile += (count[e] + TILE_ROWS - 1) / TILE_ROWS;
+    }
+    first_tile[experts] = tile;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += SORT_THREADS) {
+    const int where = first[chosen[p]] + place[p];
+    place[p] = where;
+    order[where] = p;
+  }
+  for (int e = threadIdx.x; e < experts; e += SORT_THREADS) {
+    const int n = (count[e] + TILE_ROWS - 1) / TILE_ROWS;
+    for (int i = 0; i < n; ++i) {
+      int* tile = tiles + 3 * (size_t)(first_tile[e] + i);
+      tile[0] = e;
+      tile[1] = first[e] + i * TILE_ROWS;
+      tile[2] = min(TILE_ROWS, count[e] - i * TILE_ROWS);
+    }
+  }
+  for (int i = first_tile[experts] + threadIdx.x; i < capacity; i += SORT_THREADS) {
+    tiles[3 * (size_t)i] = 0;
+    tiles[3 * (size_t)i + 1] = 0;
+    tiles[3 * (size_t)i + 2] = 0;
+  }
+}
+
+extern "C" int llmserve_sort_pairs(const int* chosen, int pairs, int experts, int* place, int* order, int* tiles,
+                                   int capacity, hipStream_t stream) {
+  if (pairs <= 0) return 0;
+  if (experts < 1 || experts > MAX_EXPERTS || capacity < (pairs + TILE_ROWS - 1) / TILE_ROWS + experts) return ERR_BAD_ARGUMENT;
+  hipLaunchKernelGGL(sort_pairs_kernel, dim3(1), dim3(SORT_THREADS), 0, stream, chosen, pairs, experts, place, order, tiles, capacity);
+  return LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------- the experts' products
+// Tile i of the list holds `rows` rows of expert e from place `first` on.  With `top` > 0 the operand's rows are the
+// tokens' (row order[place] / top of x: the first product of an expert); with top = 0 they are the places' own (the
+// second).  out[place, n] = act(sum_k row[k] * w[e, n, k]).
+template <typename TX, typename TW, typename TO>
+__global__ __launch_bounds__(256) void expert_product_kernel(const TX* __restrict__ x, const int* __restrict__ order, int top,
+                                                             const TW* __restrict__ w, int outputs, int inner,
+                                                             const int* __restrict__ tiles, TO* __restrict__ out, int activation) {
+  __shared__ float xs[TILE_ROWS * PAD_K], ws[TILE_COLS * PAD_K];
+  const int* tile = tiles + 3 * (size_t)blockIdx.y;
+  const int expert = tile[0], first = tile[1], rows = tile[2];
+  if (rows == 0) return;  // (the whole workgroup: nothing waits)
+  const int t = threadIdx.x, col0 = blockIdx.x * TILE_COLS;
+  const int load_row = t / 16, load_col = col0 + t / 4;
+  const TX* x_row = nullptr;
+  if (load_row < rows) {
+    const int place = first + load_row;
+    x_row = x + (size_t)(top > 0 ? order[place] / top : place) * inner;
+  }
+  const TW* w_row = load_col < outputs ? w + ((size_t)expert * outputs + load_col) * inner : nullptr;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  tile_product(x_row, w_row, inner, acc, xs, ws);
+  if (t / 16 >= rows) return;
+  TO* dst = out + (size_t)(first + t / 16) * outputs;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int n = col0 + t % 16 + 16 * j;
+    if (n < outputs) dst[n] = from_float<TO>(activation_of(activation, acc[j]));
+  }
+}
+
+// x, w and the first product's result are of one type (bfloat16 or float32); the second product's result is float32.
+extern "C" int llmserve_expert_product(const void* x, int is_float, const int* order, int top, const void* w, int outputs,
+                                       int inner, const int* tiles, int capacity, void* out, int out_is_float, int activation,
+                                       hipStream_t stream) {
+  if (capacity <= 0) return 0;
+  if (capacity > 65535 || outputs < 1 || inner < 1) return ERR_BAD_ARGUMENT;
+  const dim3 grid((outputs + TILE_COLS - 1) / TILE_COLS, capacity);
+  if (is_float) {
+    if (!out_is_float) return ERR_BAD_ARGUMENT;
+    hipLaunchKernelGGL((expert_product_kernel<float, float, float>), grid, dim3(256), 0, stream, (const float*)x, order, top,
+                       (const float*)w, outputs, inner, tiles, (float*)out, activation);
+  } else if (out_is_float) {
+    hipLaunchKernelGGL((expert_product_kernel<bf16_t, bf16_t, float>), grid, dim3(256), 0, stream, (const bf16_t*)x, order, top,
+                       (const bf16_t*)w, outputs, inner, tiles, (float*)out, activation);
+  } else {
+    hipLaunchKernelGGL((expert_product_kernel<bf16_t, bf16_t, bf16_t>), grid, dim3(256), 0, stream, (const bf16_t*)x, order, top,
+                       (const bf16_t*)w, outputs, inner, tiles, (bf16_t*)out, activation);
+  }
+  return LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------- the tokens' weighted sums
+// out[t] = sum_i weight[t, i] * rows[place[t * top + i]], in the order of i.
+__global__ void combine_pairs_kernel(const float* __restrict__ rows, const int* __restrict__ place, const float* __restrict__ weight,
+                                     int top, float* __restrict__ out, int width) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    float sum = 0.f;
+    for (int i = 0; i < top; ++i) sum += weight[(size_t)t * top + i] * rows[(size_t)place[(size_t)t * top + i] * width + c];
+    out[(size_t)t * width + c] = sum;
+  }
+}
+
+extern "C" int llmserve_combine_pairs(const float* rows, const int* place, const float* weight, int top, float* out, int tokens,
+                                      int width, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  hipLaunchKernelGGL(combine_pairs_kernel, dim3(tokens), dim3(256), 0, stream, rows, place, weight, top, out, width);
+  return LAUNCH_STATUS();
+}

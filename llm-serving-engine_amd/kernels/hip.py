@@ -71,6 +71,21 @@ _SIGNATURES = {
     "llmserve_argmax_static": "ppiip",
     "llmserve_sample_workspace_kib": "ii",
     "llmserve_sample": "pppppipiiip",
+    "llmserve_add_layer_norm": "ppippipiiifp",
+    "llmserve_rms_norm_columns": "piiiiipifpiiiip",
+    "llmserve_rotary_table_scaled": "pppiifp",
+    "llmserve_rotate_columns": "piiiiiiipipiiip",
+    "llmserve_join_rows": "ppippiiip",
+    "llmserve_activate": "ppiiiip",
+    "llmserve_add_gated_rows": "pppiiiip",
+    "llmserve_headwise_linear": "piiiiipiiipiiip",
+    "llmserve_route": "piipifppip",
+    "llmserve_sort_pairs": "piipppip",
+    "llmserve_expert_product": "pipipiipipiip",
+    "llmserve_combine_pairs": "pppipiip",
+    "llmserve_causal_conv": "piiiipipppippp",
+    "llmserve_gated_delta_rule": "pipppiiiippippp",
+    "llmserve_gated_head_norm": "ppiiipifiiipp",
 }
 _TYPES = {"p": ctypes.c_void_p, "i": ctypes.c_int, "f": ctypes.c_float}
 
@@ -166,8 +181,14 @@ class HipKernels:
         self._attention_bf16: dict[int, ctypes.CDLL] = {}  # by head size, compiled when a model needs it
         self._attention_f32: dict[int, ctypes.CDLL] = {}
         self._sampling = None
+        self._lazy: dict[str, ctypes.CDLL] = {}  # libraries that only some models need, compiled when one asks
 
     # ------------------------------------------------------------------ helpers
+
+    def _library_of(self, module: str) -> ctypes.CDLL:
+        if module not in self._lazy:
+            self._lazy[module] = _declared(load_module(module))
+        return self._lazy[module]
 
     @property
     def _stream(self) -> int:
@@ -241,17 +262,22 @@ class HipKernels:
         _check(status, "add_rms_norm")
         return out
 
-    def rotary_table(self, batch, inverse_frequencies: torch.Tensor) -> torch.Tensor:
-        """(cos, sin) [T, D/2, 2] float32 of position * frequency for the step's tokens.  Every
+    def rotary_table(self, batch, inverse_frequencies: torch.Tensor, magnitude: float = 1.0) -> torch.Tensor:
+        """(cos, sin) [T, D/2, 2] float32 of position * frequency for the step's tokens, times `magnitude`.  Every
         layer with the same frequencies shares it: it is computed once per step and kept on the batch."""
-        key = ("rotary_table", inverse_frequencies.data_ptr())
+        key = ("rotary_table", inverse_frequencies.data_ptr(), float(magnitude))
         table = batch.computed.get(key)
         if table is None:
             tokens, half = batch.positions.shape[0], inverse_frequencies.shape[0]
             table = self._empty((tokens, half, 2), torch.float32)
-            status = self._elementwise.llmserve_rotary_table(
-                _pointer(batch.positions), _pointer(inverse_frequencies), _pointer(table), tokens, half, self._stream
-            )
+            if magnitude != 1.0:
+                status = self._library_of("columns").llmserve_rotary_table_scaled(
+                    _pointer(batch.positions), _pointer(inverse_frequencies), _pointer(table), tokens, half, float(magnitude), self._stream
+                )
+            else:
+                status = self._elementwise.llmserve_rotary_table(
+                    _pointer(batch.positions), _pointer(inverse_frequencies), _pointer(table), tokens, half, self._stream
+                )
             _check(status, "rotary_table")
             batch.computed[key] = table
         return table
@@ -1026,6 +1052,202 @@ class HipKernels:
             return result, True
         self.rotate_and_store(qkv, layout, batch, cell, inverse_frequencies, pairing)
         return self.paged_attention(qkv, layout, batch, cell, scale, window), False
+
+    # ------------------------------------------------------------------ layer norm, runs of columns
+
+    def add_layer_norm(self, hidden, delta, weight, bias, eps: float) -> torch.Tensor:
+        rows, width = hidden.shape
+        if hidden.dtype != torch.float32 or (delta is not None and delta.dtype != torch.float32):
+            raise KernelError("add_layer_norm: the residual stream and what is added to it are float32")
+        if weight.dtype != bias.dtype or weight.shape != (width,) or bias.shape != (width,):
+            raise KernelError("add_layer_norm: weight and bias are one type and as long as a row")
+        out = self._empty((rows, width), self.dtype)
+        parts = 1 if delta is None or delta.ndim == 2 else delta.shape[0]
+        status = self._library_of("columns").llmserve_add_layer_norm(
+            _pointer(hidden), _pointer(delta), parts, _pointer(weight), _pointer(bias), _is_float(weight), _pointer(out),
+            _is_float(out), rows, width, eps, self._stream,
+        )
+        _check(status, "add_layer_norm")
+        return out
+
+    def new_rows(self, rows: int, width: int) -> torch.Tensor:
+        return self._empty((rows, width), self.dtype)
+
+    def rms_norm_columns(self, x, first: int, weight, eps: float, out=None, out_first: int = 0, copies: int = 1, copy_stride: int = 0):
+        rows, width = x.shape[0], weight.shape[0]
+        if out is None:
+            out = self._empty((rows, width), x.dtype)
+        if out.dtype != x.dtype or out.shape[0] != rows or x.ndim != 2 or out.ndim != 2:
+            raise KernelError("rms_norm_columns: input and output are rows of one type")
+        status = self._library_of("columns").llmserve_rms_norm_columns(
+            _pointer(x), _is_float(x), rows, x.shape[1], first, width, _pointer(weight), _is_float(weight), eps, _pointer(out),
+            out.shape[1], out_first, copies, copy_stride, self._stream,
+        )
+        _check(status, "rms_norm_columns")
+        return out
+
+    def rotate_columns(self, x, first: int, head_stride: int, heads: int, width: int, table, dims: int, out, out_first: int, out_head_stride: int):
+        tokens = x.shape[0]
+        if out.dtype != x.dtype or out.shape[0] != tokens or table.shape != (tokens, dims // 2, 2) or table.dtype != torch.float32:
+            raise KernelError("rotate_columns: rows of one type, and a table entry for every pair of every token")
+        status = self._library_of("columns").llmserve_rotate_columns(
+            _pointer(x), _is_float(x), tokens, x.shape[1], first, head_stride, heads, width, _pointer(table), dims, _pointer(out),
+            out.shape[1], out_first, out_head_stride, self._stream,
+        )
+        _check(status, "rotate_columns")
+        return out
+
+    def join_rows(self, hidden, delta, embedded) -> torch.Tensor:
+        rows, width = hidden.shape
+        if hidden.dtype != torch.float32 or embedded.dtype != torch.float32 or embedded.shape != hidden.shape:
+            raise KernelError("join_rows: two float32 streams of one shape")
+        out = self._empty((rows, 2 * width), self.dtype)
+        parts = 1 if delta is None or delta.ndim == 2 else delta.shape[0]
+        status = self._library_of("columns").llmserve_join_rows(
+            _pointer(hidden), _pointer(delta), parts, _pointer(embedded), _pointer(out), _is_float(out), rows, width, self._stream
+        )
+        _check(status, "join_rows")
+        return out
+
+    def activate(self, x, activation: str) -> torch.Tensor:
+        if activation not in _ACTIVATIONS:
+            raise KernelError(f"activate: no kernel applies the activation {activation!r} (known: {', '.join(_ACTIVATIONS)})")
+        out = torch.empty_like(x)
+        status = self._library_of("columns").llmserve_activate(
+            _pointer(x), _pointer(out), _is_float(x), x.shape[0], x.shape[1], _ACTIVATIONS[activation], self._stream
+        )
+        _check(status, "activate")
+        return out
+
+    def add_gated_rows(self, target, rows, gates, column: int, squash: str) -> torch.Tensor:
+        if squash != "sigmoid":
+            raise KernelError(f"add_gated_rows: no kernel squashes a gate by {squash!r}")
+        if target.dtype != torch.float32 or rows.dtype != torch.float32 or gates.dtype != torch.float32 or rows.shape != target.shape:
+            raise KernelError("add_gated_rows: float32 rows of one shape and float32 gates")
+        status = self._library_of("columns").llmserve_add_gated_rows(
+            _pointer(target), _pointer(rows), _pointer(gates), gates.shape[1], column, target.shape[0], target.shape[1], self._stream
+        )
+        _check(status, "add_gated_rows")
+        return target
+
+    # ------------------------------------------------------------------ products per head, routed experts
+
+    def prepare_headwise_linear(self, weight: torch.Tensor) -> torch.Tensor:
+        """[heads, N, K]: head h's weight."""
+        if weight.ndim != 3:
+            raise KernelError("headwise_linear: the weight is [heads, N, K]")
+        return weight.contiguous()
+
+    def headwise_linear(self, x, first: int, head_stride: int, weights, out=None, out_first: int = 0, out_head_stride: int | None = None):
+        heads, outputs, inner = weights.shape
+        rows = x.shape[0]
+        if out is None:
+            out = self._empty((rows, heads * outputs), x.dtype)
+        if x.dtype != weights.dtype or out.dtype != x.dtype or out.shape[0] != rows:
+            raise KernelError("headwise_linear: operands and result are of one type")
+        status = self._library_of("gemm_rows").llmserve_headwise_linear(
+            _pointer(x), _is_float(x), rows, x.shape[1], first, head_stride, _pointer(weights), heads, outputs, inner,
+            _pointer(out), out.shape[1], out_first, outputs if out_head_stride is None else out_head_stride, self._stream,
+        )
+        _check(status, "headwise_linear")
+        return out
+
+    def route(self, scores, experts: int, correction, top: int, scale: float, scoring: str):
+        if scoring != "sigmoid":
+            raise KernelError(f"route: no kernel scores experts by {scoring!r}")
+        if scores.dtype != torch.float32 or correction.dtype != torch.float32 or correction.shape != (experts,):
+            raise KernelError("route: float32 scores and one float32 correction an expert")
+        tokens = scores.shape[0]
+        chosen = self._empty((tokens, top), torch.int32)
+        weights = self._empty((tokens, top), torch.float32)
+        status = self._library_of("gemm_rows").llmserve_route(
+            _pointer(scores), scores.shape[1], experts, _pointer(correction), top, float(scale), _pointer(chosen), _pointer(weights),
+            tokens, self._stream,
+        )
+        _check(status, "route")
+        return chosen, weights
+
+    def prepare_experts(self, ups: list[torch.Tensor], downs: list[torch.Tensor], activation: str):
+        """The experts' weights stacked: ([experts, size, hidden], [experts, hidden, size], activation)."""
+        if activation not in _ACTIVATIONS:
+            raise KernelError(f"experts: no kernel applies the activation {activation!r} (known: {', '.join(_ACTIVATIONS)})")
+        return torch.stack(list(ups)).contiguous(), torch.stack(list(downs)).contiguous(), activation
+
+    def expert_feed_forward(self, x, experts, chosen, weights) -> torch.Tensor:
+        """sum over a token's chosen experts of weight * down(act(up x)), float32 [T, hidden].  The (token, choice)
+        pairs are sorted by expert on the device, the two products run over tiles of one expert's rows, and a last
+        kernel adds each token's rows up in the order of its choices."""
+        ups, downs, activation = experts
+        tokens, top = chosen.shape
+        count, size, hidden = ups.shape
+        if x.dtype != ups.dtype or x.shape != (tokens, hidden):
+            raise KernelError("experts: rows and weights are of one type")
+        library = self._library_of("gemm_rows")
+        pairs = tokens * top
+        capacity = -(-pairs // 16) + count
+        place = self._empty((pairs,), torch.int32)
+        order = self._empty((pairs,), torch.int32)
+        tiles = self._empty((capacity, 3), torch.int32)
+        _check(library.llmserve_sort_pairs(_pointer(chosen), pairs, count, _pointer(place), _pointer(order), _pointer(tiles), capacity, self._stream), "experts: sort")
+        inner = self._empty((pairs, size), x.dtype)
+        _check(library.llmserve_expert_product(
+            _pointer(x), _is_float(x), _pointer(order), top, _pointer(ups), size, hidden, _pointer(tiles), capacity, _pointer(inner),
+            _is_float(inner), _ACTIVATIONS[activation], self._stream), "experts: first product")
+        rows = self._empty((pairs, hidden), torch.float32)
+        _check(library.llmserve_expert_product(
+            _pointer(inner), _is_float(inner), _pointer(order), 0, _pointer(downs), hidden, size, _pointer(tiles), capacity, _pointer(rows),
+            1, -1, self._stream), "experts: second product")
+        out = self._empty((tokens, hidden), torch.float32)
+        _check(library.llmserve_combine_pairs(_pointer(rows), _pointer(place), _pointer(weights), top, _pointer(out), tokens, hidden, self._stream), "experts: sum")
+        return out
+
+    # ------------------------------------------------------------------ the gated delta rule
+
+    def causal_conv(self, x, channels: int, taps, activation: str, batch, window) -> torch.Tensor:
+        if activation != "silu":
+            raise KernelError(f"causal_conv: no kernel applies {activation!r} behind the convolution")
+        tokens = x.shape[0]
+        if taps.dtype != torch.float32 or taps.shape[0] != channels:
+            raise KernelError("causal_conv: float32 taps, a row a channel")
+        width = taps.shape[1]
+        if width > 1 and (window is None or window.dtype != torch.float32 or window.shape[1:] != (width - 1, channels)):
+            raise KernelError("causal_conv: the kept inputs are float32 [slots, taps - 1, channels]")
+        out = self._empty((tokens, channels), x.dtype)
+        status = self._library_of("delta_rule").llmserve_causal_conv(
+            _pointer(x), _is_float(x), tokens, x.shape[1], channels, _pointer(taps), width, _pointer(batch.token_sequence),
+            _pointer(batch.query_start), _pointer(batch.state_slots), batch.state_slots.shape[0], _pointer(window if width > 1 else None),
+            _pointer(out), self._stream,
+        )
+        _check(status, "causal_conv")
+        return out
+
+    def gated_delta_rule(self, mixed, controls, rate, step_bias, heads: int, kv_heads: int, dim: int, vdim: int, batch, state) -> torch.Tensor:
+        tokens = mixed.shape[0]
+        if mixed.shape[1] != 2 * kv_heads * dim + heads * vdim or controls.shape != (tokens, 2 * heads) or controls.dtype != torch.float32:
+            raise KernelError("gated_delta_rule: rows of [q | k | v] and float32 controls [b | a]")
+        if state.dtype != torch.float32 or state.shape[1:] != (heads, dim, vdim) or rate.dtype != torch.float32 or step_bias.dtype != torch.float32:
+            raise KernelError("gated_delta_rule: the state is float32 [slots, heads, dim, vdim]")
+        out = self._empty((tokens, heads * vdim), torch.float32)
+        status = self._library_of("delta_rule").llmserve_gated_delta_rule(
+            _pointer(mixed), _is_float(mixed), _pointer(controls), _pointer(rate), _pointer(step_bias), heads, kv_heads, dim, vdim,
+            _pointer(batch.query_start), _pointer(batch.state_slots), batch.state_slots.shape[0], _pointer(state), _pointer(out), self._stream,
+        )
+        _check(status, "gated_delta_rule")
+        return out
+
+    def gated_head_norm(self, read, gates, gate_first: int, weight, eps: float, heads: int, vdim: int, activation: str) -> torch.Tensor:
+        if activation != "silu":
+            raise KernelError(f"gated_head_norm: no kernel gates by {activation!r}")
+        tokens = read.shape[0]
+        if read.dtype != torch.float32 or read.shape[1] != heads * vdim or weight.shape != (vdim,):
+            raise KernelError("gated_head_norm: a float32 read-out [T, heads * vdim] and a weight of vdim")
+        out = self._empty((tokens, heads * vdim), gates.dtype)
+        status = self._library_of("delta_rule").llmserve_gated_head_norm(
+            _pointer(read), _pointer(gates), _is_float(gates), gates.shape[1], gate_first, _pointer(weight), _is_float(weight), eps,
+            tokens, heads, vdim, _pointer(out), self._stream,
+        )
+        _check(status, "gated_head_norm")
+        return out
 
     # ------------------------------------------------------------------ sampling
 

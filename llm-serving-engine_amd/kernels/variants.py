@@ -11,6 +11,9 @@ DEFAULT_VARIANTS: dict[str, list[dict[str, object]]] = {
     "gemm_bf16": [{}],
     "attention_generic": [{}],
     "sampling": [{}],
+    "columns": [{}],
+    "gemm_rows": [{}],
+    "delta_rule": [{}],
     # head sizes of the tests' models and kernel tests, and of the benchmark
     "attention_bf16": [{"HEAD_DIM": d} for d in (16, 32, 48, 64, 80, 96, 112, 128, 144, 160, 192, 256)],
     "attention_f32": [{"HEAD_DIM": d} for d in (16, 32, 48, 64, 80, 96, 112, 128, 144, 160, 192, 256)],
