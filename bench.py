@@ -65,7 +65,7 @@ def parse() -> argparse.Namespace:
                         help="leave out decoding at contexts of 8k and 30k (batch 8) and 4k (batch 64), and the long prompts")
     parser.add_argument("--skip-other-models", action="store_true",
                         help="leave out the float32 run and the 7B and 32B layer sizes")
-    parser.add_argument("--op", choices=("decode-attention", "prefill-attention"), default=None,
+    parser.add_argument("--op", choices=("decode-attention", "prefill-attention", "dafutar"), default=None,
                         help="measure one operation alone instead, as the reference's kernel benchmark does")
     return parser.parse_args()
 
@@ -414,6 +414,8 @@ def main() -> int:
         return decode_attention_table(args)
     if args.op == "prefill-attention":
         return prefill_attention_table(args)
+    if args.op == "dafutar":
+        return dafutar_table(args)
 
     import torch
 
@@ -539,6 +541,43 @@ def main() -> int:
         "points": points,
     }
     print(json.dumps(record))
+    return 0
+
+
+def dafutar_table(args) -> int:
+    """The Dafutar decoder (layers of the gated delta rule and of latent attention, dense and routed feed-forwards) at
+    two layer sizes beside a Qwen2 of the same width, number of layer runs and vocabulary: decoding at `--batch`
+    requests after `--prompt-len`-token prompts and the prefill of a `--prefill-len`-token prompt, random weights.
+    One JSON line; the default run of this file is not touched."""
+    import torch
+
+    pairs = [
+        ("w1536", ROOT / "configs" / "dafutar-w1536.json", ROOT / "configs" / "qwen2-w1536-12-layers.json"),
+        ("w3584", ROOT / "configs" / "dafutar-w3584.json", ROOT / "configs" / "qwen2-w3584-4-layers.json"),
+    ]
+    steps, warmup, repeats = max(1, min(args.steps, 64)), min(args.warmup, 8), min(max(1, args.repeats), 3)
+    shape = (args.batch, args.prompt_len, output_tokens(args.batch, args.prompt_len, steps, warmup))
+    points: dict = {}
+    for tag, *paths in pairs:
+        for name, path in zip(("dafutar", "qwen2"), paths):
+            bench = Bench(str(path), args.dtype, args.seed, library_products=not args.own_products, shapes=[shape], prefill_tokens=args.prefill_len)
+            decode = bench.decode(args.batch, args.prompt_len, steps, warmup, repeats)
+            prefill = bench.prefill(args.prefill_len, repeats=3)
+            key = f"{name}_{tag}"
+            put(points, f"{key}_decode_b{args.batch}", decode)
+            points[f"{key}_prefill"] = prefill["value"]
+            points[f"{key}_prefill_ms"] = prefill["ms"]
+            points[f"{key}_layer_runs"] = len(bench.spec.run_order)
+            points[f"{key}_weight_mb"] = round(bench.weight_bytes / 1e6, 1)
+            points[f"{key}_cache_bytes_per_token"] = bench.kv_bytes_per_token
+            bench.close()
+            del bench
+            torch.cuda.empty_cache()
+    print(json.dumps({
+        "metric": f"decode tok/s at batch {args.batch} and prefill tok/s of {args.prefill_len} tokens, Dafutar beside Qwen2 at equal sizes",
+        "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "dtype": args.dtype,
+        "data": "synthetic: seeded random weights, uniform random token ids", "points": points,
+    }))
     return 0
 
 
