@@ -82,68 +82,118 @@ extern "C" int llmserve_causal_conv(const void* x, int is_float, int tokens, int
 //   q <- q / sqrt(sum q^2 + 1e-6) * dim^-1/2,   k <- k / sqrt(sum k^2 + 1e-6),
 //   beta = sigmoid(b),   g = exp(-exp(rate_h) * softplus(a + step_bias_h)),
 //   S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q            (S [dim, vdim], float32)
-// Column j of S (the state of value dimension j) never meets another column, so a lane owns one column and keeps
-// its dim numbers in registers for all the tokens of the request's step; a wave owns 64 columns of one (request,
-// head), and the lanes share q and k, which each lane loads a piece of and all read lane by lane.  The state comes
-// from state[slot, h] ([dim, vdim], columns side by side) and goes back there after the step's last token.
-template <typename T, int PIECES>  // PIECES * 64 >= dim
+// Column j of S (the state of value dimension j) never meets another column.  A wave owns 16 columns of one (request,
+// head): four neighbouring lanes share a column, each keeping a quarter of its rows (ROWS numbers) in registers for all
+// the tokens of the request's step, and the two sums over a column's rows end with two exchanges between those lanes.
+// The tokens are walked in runs of RUN: first the wave brings the run's q, k, v and controls from memory (all loads
+// under way together: a token by itself would wait for memory every time), makes q and k unit vectors and the decays
+// and betas (lane c those of the run's token c), and leaves them in LDS; then it walks the run token by token out of
+// LDS and registers alone.  The state comes from state[slot, h] ([dim, vdim], columns side by side) and goes back there
+// after the step's last token.
+#define RUN 16
+#define COLUMNS 16
+template <typename T, int ROWS>  // 4 * ROWS >= dim; ROWS a multiple of 4
 __global__ __launch_bounds__(64) void gated_delta_rule_kernel(const T* __restrict__ mixed, const float* __restrict__ controls,
                                                               const float* __restrict__ rate, const float* __restrict__ step_bias,
                                                               int heads, int kv_heads, int dim, int vdim,
                                                               const int* __restrict__ start, const int* __restrict__ slots,
                                                               float* __restrict__ state, float* __restrict__ out) {
+  constexpr int PADDED = 4 * ROWS, PIECES = (PADDED + WAVE - 1) / WAVE, LINE = 4 * (ROWS + 4);  // (a quarter's rows, then 4 floats: banks)
+  __shared__ __attribute__((aligned(16))) float keys[RUN][LINE], queries[RUN][LINE];
+  __shared__ float decays[RUN], betas[RUN];
   const int b = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
-  const int column = blockIdx.z * WAVE + lane;
+  const int column = blockIdx.z * COLUMNS + lane / 4, quarter = lane % 4;
   const bool owns = column < vdim;
   const int first = start[b], last = start[b + 1];
   if (last <= first) return;
   const int kv_head = head / (heads / kv_heads);
   const int row_width = 2 * kv_heads * dim + heads * vdim;
   float* mine = state + ((size_t)slots[b] * heads + head) * dim * vdim + column;
-  float S[PIECES * WAVE];
+  float S[ROWS];
 #pragma unroll
-  for (int i = 0; i < PIECES * WAVE; ++i) S[i] = (owns && i < dim) ? mine[(size_t)i * vdim] : 0.f;
+  for (int r = 0; r < ROWS; ++r) {
+    const int i = quarter * ROWS + r;
+    S[r] = (owns && i < dim) ? mine[(size_t)i * vdim] : 0.f;
+  }
   const float speed = expf(rate[head]), bias = step_bias[head];
   const float q_scale = rsqrtf((float)dim);
-  for (int t = first; t < last; ++t) {
-    const T* row = mixed + (size_t)t * row_width;
-    float q[PIECES], k[PIECES];
-    float q_squares = 0.f, k_squares = 0.f;
+  for (int t0 = first; t0 < last; t0 += RUN) {
+    float q[RUN][PIECES], k[RUN][PIECES], v[RUN];
 #pragma unroll
-    for (int p = 0; p < PIECES; ++p) {
-      const int i = p * WAVE + lane;
-      q[p] = i < dim ? to_float(row[kv_head * dim + i]) : 0.f;
-      k[p] = i < dim ? to_float(row[(kv_heads + kv_head) * dim + i]) : 0.f;
-      q_squares += q[p] * q[p];
-      k_squares += k[p] * k[p];
+    for (int c = 0; c < RUN; ++c) {
+      const bool valid = t0 + c < last;
+      const T* row = mixed + (size_t)(valid ? t0 + c : t0) * row_width;
+#pragma unroll
+      for (int p = 0; p < PIECES; ++p) {
+        const int i = p * WAVE + lane;
+        q[c][p] = (valid && i < dim) ? to_float(row[kv_head * dim + i]) : 0.f;
+        k[c][p] = (valid && i < dim) ? to_float(row[(kv_heads + kv_head) * dim + i]) : 0.f;
+      }
+      v[c] = (valid && owns) ? to_float(row[2 * kv_heads * dim + head * vdim + column]) : 0.f;
     }
-    const float q_unit = q_scale / sqrtf(wave_sum(q_squares) + 1e-6f), k_unit = 1.f / sqrtf(wave_sum(k_squares) + 1e-6f);
-#pragma unroll
-    for (int p = 0; p < PIECES; ++p) { q[p] *= q_unit; k[p] *= k_unit; }
-    const float v = owns ? to_float(row[2 * kv_heads * dim + head * vdim + column]) : 0.f;
-    const float b_in = controls[(size_t)t * 2 * heads + head], a_in = controls[(size_t)t * 2 * heads + heads + head] + bias;
-    const float beta = 1.f / (1.f + expf(-b_in));
-    const float softplus = a_in > 20.f ? a_in : log1pf(expf(a_in));
-    const float g = expf(-speed * softplus);
-    float seen = 0.f;  // (g S)^T k
-#pragma unroll
-    for (int i = 0; i < PIECES * WAVE; ++i) {
-      S[i] *= g;
-      seen += S[i] * __shfl(k[i / WAVE], i % WAVE, WAVE);
+    if (lane < RUN && t0 + lane < last) {
+      const size_t at = (size_t)(t0 + lane) * 2 * heads;
+      const float b_in = controls[at + head], a_in = controls[at + heads + head] + bias;
+      const float softplus = a_in > 20.f ? a_in : log1pf(expf(a_in));
+      betas[lane] = 1.f / (1.f + expf(-b_in));
+      decays[lane] = expf(-speed * softplus);
     }
-    const float u = beta * (v - seen);
-    float read = 0.f;
 #pragma unroll
-    for (int i = 0; i < PIECES * WAVE; ++i) {
-      S[i] += __shfl(k[i / WAVE], i % WAVE, WAVE) * u;
-      read += S[i] * __shfl(q[i / WAVE], i % WAVE, WAVE);
+    for (int c = 0; c < RUN; ++c) {
+      float q_squares = 0.f, k_squares = 0.f;
+#pragma unroll
+      for (int p = 0; p < PIECES; ++p) {
+        q_squares += q[c][p] * q[c][p];
+        k_squares += k[c][p] * k[c][p];
+      }
+      const float q_unit = q_scale / sqrtf(wave_sum(q_squares) + 1e-6f), k_unit = 1.f / sqrtf(wave_sum(k_squares) + 1e-6f);
+#pragma unroll
+      for (int p = 0; p < PIECES; ++p) {
+        const int i = p * WAVE + lane;
+        if (i < PADDED) {
+          const int where = (i / ROWS) * (ROWS + 4) + i % ROWS;
+          queries[c][where] = q[c][p] * q_unit;
+          keys[c][where] = k[c][p] * k_unit;
+        }
+      }
     }
-    if (owns) out[(size_t)t * heads * vdim + head * vdim + column] = read;
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < RUN; ++c) {
+      if (t0 + c < last) {
+        const float g = decays[c], beta = betas[c];
+        const float4* key = (const float4*)&keys[c][quarter * (ROWS + 4)];
+        const float4* query = (const float4*)&queries[c][quarter * (ROWS + 4)];
+        float seen = 0.f;  // (g S)^T k, this lane's rows
+#pragma unroll
+        for (int r = 0; r < ROWS; r += 4) {
+          const float4 kk = key[r / 4];
+          S[r] *= g; S[r + 1] *= g; S[r + 2] *= g; S[r + 3] *= g;
+          seen += S[r] * kk.x; seen += S[r + 1] * kk.y; seen += S[r + 2] * kk.z; seen += S[r + 3] * kk.w;
+        }
+        seen += __shfl_xor(seen, 1, WAVE);
+        seen += __shfl_xor(seen, 2, WAVE);
+        const float u = beta * (v[c] - seen);
+        float read = 0.f;
+#pragma unroll
+        for (int r = 0; r < ROWS; r += 4) {
+          const float4 kk = key[r / 4], qq = query[r / 4];
+          S[r] += kk.x * u; S[r + 1] += kk.y * u; S[r + 2] += kk.z * u; S[r + 3] += kk.w * u;
+          read += S[r] * qq.x; read += S[r + 1] * qq.y; read += S[r + 2] * qq.z; read += S[r + 3] * qq.w;
+        }
+        read += __shfl_xor(read, 1, WAVE);
+        read += __shfl_xor(read, 2, WAVE);
+        if (owns && quarter == 0) out[(size_t)(t0 + c) * heads * vdim + head * vdim + column] = read;
+      }
+    }
+    __syncthreads();  // the next run overwrites what this one read
   }
   if (owns) {
 #pragma unroll
-    for (int i = 0; i < PIECES * WAVE; ++i)
-      if (i < dim) mine[(size_t)i * vdim] = S[i];
+    for (int r = 0; r < ROWS; ++r) {
+      const int i = quarter * ROWS + r;
+      if (i < dim) mine[(size_t)i * vdim] = S[r];
+    }
   }
 }
 
@@ -151,16 +201,15 @@ extern "C" int llmserve_gated_delta_rule(const void* mixed, int is_float, const 
                                          const float* step_bias, int heads, int kv_heads, int dim, int vdim, const int* start,
                                          const int* slots, int requests, float* state, float* out, hipStream_t stream) {
   if (requests <= 0) return 0;
-  if (heads < 1 || kv_heads < 1 || heads % kv_heads || dim < 1 || dim > 4 * WAVE || vdim < 1 || heads > 65535) return ERR_BAD_ARGUMENT;
-  const dim3 grid(requests, heads, (vdim + WAVE - 1) / WAVE);
-  const int pieces = (dim + WAVE - 1) / WAVE;
-#define LAUNCH_RULE(TYPE, PIECES)                                                                                              \
-  hipLaunchKernelGGL((gated_delta_rule_kernel<TYPE, PIECES>), grid, dim3(WAVE), 0, stream, (const TYPE*)mixed, controls, rate, \
+  if (heads < 1 || kv_heads < 1 || heads % kv_heads || dim < 1 || dim > 256 || vdim < 1 || heads > 65535) return ERR_BAD_ARGUMENT;
+  const dim3 grid(requests, heads, (vdim + COLUMNS - 1) / COLUMNS);
+#define LAUNCH_RULE(TYPE, ROWS)                                                                                              \
+  hipLaunchKernelGGL((gated_delta_rule_kernel<TYPE, ROWS>), grid, dim3(WAVE), 0, stream, (const TYPE*)mixed, controls, rate, \
                      step_bias, heads, kv_heads, dim, vdim, start, slots, state, out)
   if (is_float) {
-    if (pieces == 1) LAUNCH_RULE(float, 1); else if (pieces == 2) LAUNCH_RULE(float, 2); else LAUNCH_RULE(float, 4);
+    if (dim <= 32) LAUNCH_RULE(float, 8); else if (dim <= 64) LAUNCH_RULE(float, 16); else if (dim <= 128) LAUNCH_RULE(float, 32); else LAUNCH_RULE(float, 64);
   } else {
-    if (pieces == 1) LAUNCH_RULE(bf16_t, 1); else if (pieces == 2) LAUNCH_RULE(bf16_t, 2); else LAUNCH_RULE(bf16_t, 4);
+    if (dim <= 32) LAUNCH_RULE(bf16_t, 8); else if (dim <= 64) LAUNCH_RULE(bf16_t, 16); else if (dim <= 128) LAUNCH_RULE(bf16_t, 32); else LAUNCH_RULE(bf16_t, 64);
   }
 #undef LAUNCH_RULE
   return LAUNCH_STATUS();

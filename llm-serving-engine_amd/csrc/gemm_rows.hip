@@ -1,8 +1,12 @@
 // Products whose rows or weights are chosen per tile: a product per head over a run of a row's columns, and the
 // products of routed experts over rows that were sorted by expert on the device.  One core: a workgroup of 256
 // threads makes a 16 x 64 tile of the result, K in steps of 32 through LDS, float32 arithmetic and sums in the
-// order of k whatever the batch holds.  Operands are bfloat16 or float32.
+// order of k whatever the batch holds.  Operands are bfloat16 or float32.  bfloat16 operands whose K is a multiple
+// of 32 and whose rows begin at multiples of 8 elements go to the matrix cores instead (the second core below).
 #include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define TILE_ROWS 16
 #define TILE_COLS 64
@@ -53,6 +57,117 @@ __device__ __forceinline__ void tile_product(const TX* x_row, const TW* w_row, i
   }
 }
 
+// The matrix-core form.  A wave makes NT x MT tiles of v_mfma_f32_16x16x32_bf16: weight rows are the A operand (lane l
+// holds row l % 16, k = (l / 16) * 8 .. + 8 of a 32-wide step), the operand's rows the B operand (lane l: row l % 16, the
+// same k), both straight from memory in 16-byte loads, and the result tile D[n][m] leaves four consecutive n of row
+// l % 16 in lane l.  `w_row[s]` and `x_row[t]` are the lane's rows already moved to its k (null: zeros).
+template <int NT, int MT>
+__device__ __forceinline__ void tile_product_mfma(const bf16_t* const (&w_row)[NT], const bf16_t* const (&x_row)[MT], int inner,
+                                                  f32x4 (&acc)[NT][MT]) {
+  const bf16x8 zero = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll 2
+  for (int k0 = 0; k0 < inner; k0 += 32) {
+    bf16x8 a[NT], b[MT];
+#pragma unroll
+    for (int s = 0; s < NT; ++s) a[s] = w_row[s] ? *(const bf16x8*)(w_row[s] + k0) : zero;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) b[t] = x_row[t] ? *(const bf16x8*)(x_row[t] + k0) : zero;
+#pragma unroll
+    for (int s = 0; s < NT; ++s)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s], b[t], acc[s][t], 0, 0, 0);
+  }
+}
+
+// A workgroup of four waves makes 16 MT rows by 64 NT columns, wave v the columns 16 NT v .. + 16 NT.
+template <int NT, int MT>
+__global__ __launch_bounds__(256) void headwise_mfma_kernel(const bf16_t* __restrict__ x, int x_stride, int first, int head_stride,
+                                                            const bf16_t* __restrict__ w, int outputs, int inner,
+                                                            bf16_t* __restrict__ out, int out_stride, int out_first,
+                                                            int out_head_stride, int rows) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+  const int head = blockIdx.z, row0 = blockIdx.y * 16 * MT, col0 = (blockIdx.x * 4 + wave) * 16 * NT;
+  if (col0 >= outputs) return;
+  const bf16_t* w_row[NT];
+  const bf16_t* x_row[MT];
+#pragma unroll
+  for (int s = 0; s < NT; ++s) {
+    const int n = col0 + s * 16 + r;
+    w_row[s] = n < outputs ? w + ((size_t)head * outputs + n) * inner + g * 8 : nullptr;
+  }
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = row0 + t * 16 + r;
+    x_row[t] = m < rows ? x + (size_t)m * x_stride + first + (size_t)head * head_stride + g * 8 : nullptr;
+  }
+  f32x4 acc[NT][MT];
+#pragma unroll
+  for (int s = 0; s < NT; ++s)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[s][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  tile_product_mfma<NT, MT>(w_row, x_row, inner, acc);
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = row0 + t * 16 + r;
+    if (m >= rows) continue;
+    bf16_t* dst = out + (size_t)m * out_stride + out_first + (size_t)head * out_head_stride;
+#pragma unroll
+    for (int s = 0; s < NT; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = col0 + s * 16 + g * 4 + i;
+        if (n < outputs) dst[n] = (bf16_t)acc[s][t][i];
+      }
+  }
+}
+
+template <int NT, int MT, typename TO>
+__global__ __launch_bounds__(256) void expert_product_mfma_kernel(const bf16_t* __restrict__ x, const int* __restrict__ order, int top,
+                                                                  const bf16_t* __restrict__ w, int outputs, int inner,
+                                                                  const int* __restrict__ tiles, TO* __restrict__ out, int activation) {
+  const int* tile = tiles + 3 * (size_t)blockIdx.y;
+  const int expert = tile[0], first = tile[1], rows = tile[2];
+  if (rows == 0) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+  const int col0 = (blockIdx.x * 4 + wave) * 16 * NT;
+  if (col0 >= outputs) return;
+  const bf16_t* w_row[NT];
+  const bf16_t* x_row[MT];
+#pragma unroll
+  for (int s = 0; s < NT; ++s) {
+    const int n = col0 + s * 16 + r;
+    w_row[s] = n < outputs ? w + ((size_t)expert * outputs + n) * inner + g * 8 : nullptr;
+  }
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = t * 16 + r;
+    x_row[t] = nullptr;
+    if (m < rows) {
+      const int place = first + m;
+      x_row[t] = x + (size_t)(top > 0 ? order[place] / top : place) * inner + g * 8;
+    }
+  }
+  f32x4 acc[NT][MT];
+#pragma unroll
+  for (int s = 0; s < NT; ++s)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[s][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  tile_product_mfma<NT, MT>(w_row, x_row, inner, acc);
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = t * 16 + r;
+    if (m >= rows) continue;
+    TO* dst = out + (size_t)(first + m) * outputs;
+#pragma unroll
+    for (int s = 0; s < NT; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = col0 + s * 16 + g * 4 + i;
+        if (n < outputs) dst[n] = from_float<TO>(activation_of(activation, acc[s][t][i]));
+      }
+  }
+}
+
 // ---------------------------------------------------------------------------- a product per head
 // out[t, out_first + h * out_head_stride + n] = sum_k x[t, first + h * head_stride + k] * w[h, n, k]
 template <typename T>
@@ -86,6 +201,21 @@ extern "C" int llmserve_headwise_linear(const void* x, int is_float, int rows, i
     return ERR_BAD_ARGUMENT;
   const dim3 grid((outputs + TILE_COLS - 1) / TILE_COLS, (rows + TILE_ROWS - 1) / TILE_ROWS, heads);
   if (grid.y > 65535) return ERR_BAD_ARGUMENT;
+  if (!is_float && inner % 32 == 0 && x_stride % 8 == 0 && first % 8 == 0 && head_stride % 8 == 0) {
+    // the matrix cores: four row tiles a wave for many rows, one for a few; as many column tiles as the columns need
+    const int mt = rows > 16 ? 4 : 1, nt = outputs <= 64 ? 1 : outputs <= 128 ? 2 : 4;
+    const dim3 cores((outputs + 64 * nt - 1) / (64 * nt), (rows + 16 * mt - 1) / (16 * mt), heads);
+#define LAUNCH_HEADWISE(NT, MT)                                                                                                 \
+  hipLaunchKernelGGL((headwise_mfma_kernel<NT, MT>), cores, dim3(256), 0, stream, (const bf16_t*)x, x_stride, first, head_stride, \
+                     (const bf16_t*)w, outputs, inner, (bf16_t*)out, out_stride, out_first, out_head_stride, rows)
+    if (mt == 4) {
+      if (nt == 1) LAUNCH_HEADWISE(1, 4); else if (nt == 2) LAUNCH_HEADWISE(2, 4); else LAUNCH_HEADWISE(4, 4);
+    } else {
+      if (nt == 1) LAUNCH_HEADWISE(1, 1); else if (nt == 2) LAUNCH_HEADWISE(2, 1); else LAUNCH_HEADWISE(4, 1);
+    }
+#undef LAUNCH_HEADWISE
+    return LAUNCH_STATUS();
+  }
   if (is_float)
     hipLaunchKernelGGL(headwise_kernel<float>, grid, dim3(256), 0, stream, (const float*)x, x_stride, first, head_stride,
                        (const float*)w, outputs, inner, (float*)out, out_stride, out_first, out_head_stride, rows);
@@ -132,13 +262,13 @@ extern "C" int llmserve_route(const float* z, int z_stride, int experts, const f
 // ---------------------------------------------------------------------------- sorting the (token, choice) pairs by expert
 // One workgroup.  place[p] is where pair p = t * top + i stands in the order by expert (the order within an expert is
 // whichever the counting gave: every row is computed by itself, so results do not depend on it); order[place[p]] = p.
-// The tiles of the grouped products, TILE_ROWS rows of one expert each: tile[i] = (expert, first place, rows); there is
-// room for ceil(pairs / TILE_ROWS) + experts of them, and those not needed have no rows.
+// The tiles of the grouped products, up to `tile_rows` rows of one expert each: tile[i] = (expert, first place, rows);
+// there is room for ceil(pairs / tile_rows) + experts of them, and those not needed have no rows.
 #define SORT_THREADS 1024
 #define MAX_EXPERTS 1024
 __global__ __launch_bounds__(SORT_THREADS) void sort_pairs_kernel(const int* __restrict__ chosen, int pairs, int experts,
                                                                   int* __restrict__ place, int* __restrict__ order,
-                                                                  int* __restrict__ tiles, int capacity) {
+                                                                  int* __restrict__ tiles, int capacity, int tile_rows) {
   __shared__ int count[MAX_EXPERTS], first[MAX_EXPERTS], first_tile[MAX_EXPERTS + 1];
   for (int e = threadIdx.x; e < experts; e += SORT_THREADS) count[e] = 0;
   __syncthreads();
@@ -150,7 +280,7 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_pairs_kernel(const int* __r
       first[e] = rows;
       first_tile[e] = tile;
       rows += count[e];
-      tile += (count[e] + TILE_ROWS - 1) / TILE_ROWS;
+      tile += (count[e] + tile_rows - 1) / tile_rows;
     }
     first_tile[experts] = tile;
   }
@@ -161,12 +291,12 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_pairs_kernel(const int* __r
     order[where] = p;
   }
   for (int e = threadIdx.x; e < experts; e += SORT_THREADS) {
-    const int n = (count[e] + TILE_ROWS - 1) / TILE_ROWS;
+    const int n = (count[e] + tile_rows - 1) / tile_rows;
     for (int i = 0; i < n; ++i) {
       int* tile = tiles + 3 * (size_t)(first_tile[e] + i);
       tile[0] = e;
-      tile[1] = first[e] + i * TILE_ROWS;
-      tile[2] = min(TILE_ROWS, count[e] - i * TILE_ROWS);
+      tile[1] = first[e] + i * tile_rows;
+      tile[2] = min(tile_rows, count[e] - i * tile_rows);
     }
   }
   for (int i = first_tile[experts] + threadIdx.x; i < capacity; i += SORT_THREADS) {
@@ -177,10 +307,13 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_pairs_kernel(const int* __r
 }
 
 extern "C" int llmserve_sort_pairs(const int* chosen, int pairs, int experts, int* place, int* order, int* tiles,
-                                   int capacity, hipStream_t stream) {
+                                   int capacity, int tile_rows, hipStream_t stream) {
   if (pairs <= 0) return 0;
-  if (experts < 1 || experts > MAX_EXPERTS || capacity < (pairs + TILE_ROWS - 1) / TILE_ROWS + experts) return ERR_BAD_ARGUMENT;
-  hipLaunchKernelGGL(sort_pairs_kernel, dim3(1), dim3(SORT_THREADS), 0, stream, chosen, pairs, experts, place, order, tiles, capacity);
+  if (experts < 1 || experts > MAX_EXPERTS || (tile_rows != 16 && tile_rows != 64) ||
+      capacity < (pairs + tile_rows - 1) / tile_rows + experts)
+    return ERR_BAD_ARGUMENT;
+  hipLaunchKernelGGL(sort_pairs_kernel, dim3(1), dim3(SORT_THREADS), 0, stream, chosen, pairs, experts, place, order, tiles, capacity,
+                     tile_rows);
   return LAUNCH_STATUS();
 }
 
@@ -216,11 +349,35 @@ __global__ __launch_bounds__(256) void expert_product_kernel(const TX* __restric
 }
 
 // x, w and the first product's result are of one type (bfloat16 or float32); the second product's result is float32.
+// `tile_rows` is what the tiles were made for: 16, or 64 (bfloat16 with a K in steps of 32 only: the matrix cores).
 extern "C" int llmserve_expert_product(const void* x, int is_float, const int* order, int top, const void* w, int outputs,
-                                       int inner, const int* tiles, int capacity, void* out, int out_is_float, int activation,
-                                       hipStream_t stream) {
+                                       int inner, const int* tiles, int capacity, int tile_rows, void* out, int out_is_float,
+                                       int activation, hipStream_t stream) {
   if (capacity <= 0) return 0;
   if (capacity > 65535 || outputs < 1 || inner < 1) return ERR_BAD_ARGUMENT;
+  if (!is_float && inner % 32 == 0) {
+    const int nt = outputs <= 64 ? 1 : outputs <= 128 ? 2 : 4;
+    const dim3 cores((outputs + 64 * nt - 1) / (64 * nt), capacity);
+#define LAUNCH_EXPERTS(NT, MT)                                                                                                  \
+  do {                                                                                                                          \
+    if (out_is_float)                                                                                                           \
+      hipLaunchKernelGGL((expert_product_mfma_kernel<NT, MT, float>), cores, dim3(256), 0, stream, (const bf16_t*)x, order, top, \
+                         (const bf16_t*)w, outputs, inner, tiles, (float*)out, activation);                                     \
+    else                                                                                                                        \
+      hipLaunchKernelGGL((expert_product_mfma_kernel<NT, MT, bf16_t>), cores, dim3(256), 0, stream, (const bf16_t*)x, order, top, \
+                         (const bf16_t*)w, outputs, inner, tiles, (bf16_t*)out, activation);                                    \
+  } while (0)
+    if (tile_rows == 64) {
+      if (nt == 1) LAUNCH_EXPERTS(1, 4); else if (nt == 2) LAUNCH_EXPERTS(2, 4); else LAUNCH_EXPERTS(4, 4);
+    } else if (tile_rows == 16) {
+      if (nt == 1) LAUNCH_EXPERTS(1, 1); else if (nt == 2) LAUNCH_EXPERTS(2, 1); else LAUNCH_EXPERTS(4, 1);
+    } else {
+      return ERR_BAD_ARGUMENT;
+    }
+#undef LAUNCH_EXPERTS
+    return LAUNCH_STATUS();
+  }
+  if (tile_rows != TILE_ROWS) return ERR_BAD_ARGUMENT;
   const dim3 grid((outputs + TILE_COLS - 1) / TILE_COLS, capacity);
   if (is_float) {
     if (!out_is_float) return ERR_BAD_ARGUMENT;

@@ -80,8 +80,8 @@ _SIGNATURES = {
     "llmserve_add_gated_rows": "pppiiiip",
     "llmserve_headwise_linear": "piiiiipiiipiiip",
     "llmserve_route": "piipifppip",
-    "llmserve_sort_pairs": "piipppip",
-    "llmserve_expert_product": "pipipiipipiip",
+    "llmserve_sort_pairs": "piipppiip",
+    "llmserve_expert_product": "pipipiipiipiip",
     "llmserve_combine_pairs": "pppipiip",
     "llmserve_causal_conv": "piiiipipppippp",
     "llmserve_gated_delta_rule": "pipppiiiippippp",
@@ -1184,18 +1184,21 @@ class HipKernels:
             raise KernelError("experts: rows and weights are of one type")
         library = self._library_of("gemm_rows")
         pairs = tokens * top
-        capacity = -(-pairs // 16) + count
+        # tiles of 64 rows for the matrix cores where an expert has that many rows or so, else of 16
+        on_cores = x.dtype == torch.bfloat16 and hidden % 32 == 0 and size % 32 == 0
+        tile_rows = 64 if on_cores and pairs >= 32 * count else 16
+        capacity = -(-pairs // tile_rows) + count
         place = self._empty((pairs,), torch.int32)
         order = self._empty((pairs,), torch.int32)
         tiles = self._empty((capacity, 3), torch.int32)
-        _check(library.llmserve_sort_pairs(_pointer(chosen), pairs, count, _pointer(place), _pointer(order), _pointer(tiles), capacity, self._stream), "experts: sort")
+        _check(library.llmserve_sort_pairs(_pointer(chosen), pairs, count, _pointer(place), _pointer(order), _pointer(tiles), capacity, tile_rows, self._stream), "experts: sort")
         inner = self._empty((pairs, size), x.dtype)
         _check(library.llmserve_expert_product(
-            _pointer(x), _is_float(x), _pointer(order), top, _pointer(ups), size, hidden, _pointer(tiles), capacity, _pointer(inner),
+            _pointer(x), _is_float(x), _pointer(order), top, _pointer(ups), size, hidden, _pointer(tiles), capacity, tile_rows, _pointer(inner),
             _is_float(inner), _ACTIVATIONS[activation], self._stream), "experts: first product")
         rows = self._empty((pairs, hidden), torch.float32)
         _check(library.llmserve_expert_product(
-            _pointer(inner), _is_float(inner), _pointer(order), 0, _pointer(downs), hidden, size, _pointer(tiles), capacity, _pointer(rows),
+            _pointer(inner), _is_float(inner), _pointer(order), 0, _pointer(downs), hidden, size, _pointer(tiles), capacity, tile_rows, _pointer(rows),
             1, -1, self._stream), "experts: second product")
         out = self._empty((tokens, hidden), torch.float32)
         _check(library.llmserve_combine_pairs(_pointer(rows), _pointer(place), _pointer(weights), top, _pointer(out), tokens, hidden, self._stream), "experts: sum")

@@ -97,18 +97,23 @@ def test_rotate_columns(kernels, dtype, dims, width):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("rows,heads,outputs,inner", [(1, 3, 5, 7), (19, 6, 128, 64), (70, 2, 70, 100)])
-def test_headwise_linear(kernels, dtype, rows, heads, outputs, inner):
+@pytest.mark.parametrize("rows,heads,outputs,inner,gap", [
+    (1, 3, 5, 7, 3), (19, 6, 128, 64, 3), (70, 2, 70, 100, 3),
+    # rows that begin at multiples of eight elements and a K in steps of 32: in bfloat16 the matrix cores
+    (3, 5, 192, 128, 8), (150, 3, 40, 64, 16), (33, 2, 300, 96, 0),
+])
+def test_headwise_linear(kernels, dtype, rows, heads, outputs, inner, gap):
     torch.manual_seed(rows)
-    stride = inner + 3
-    x = torch.randn(rows, 4 + heads * stride).to(dtype)
+    stride = inner + gap
+    x = torch.randn(rows, 8 + heads * stride).to(dtype)
     weight = (torch.randn(heads, outputs, inner) / inner**0.5).to(dtype)
     plain = TorchKernels(dtype)
     prepared = kernels[dtype].prepare_headwise_linear(gpu(weight))
-    close(kernels[dtype].headwise_linear(gpu(x), 4, stride, prepared), plain.headwise_linear(x, 4, stride, weight.float()), dtype)
+    first = 8 if gap % 8 == 0 else 4
+    close(kernels[dtype].headwise_linear(gpu(x), first, stride, prepared), plain.headwise_linear(x, first, stride, weight.float()), dtype)
     out, want = torch.zeros(rows, 2 + heads * (outputs + 6)).to(dtype), torch.zeros(rows, 2 + heads * (outputs + 6)).to(dtype)
-    plain.headwise_linear(x, 4, stride, weight.float(), out=want, out_first=2, out_head_stride=outputs + 6)
-    got = kernels[dtype].headwise_linear(gpu(x), 4, stride, prepared, out=gpu(out), out_first=2, out_head_stride=outputs + 6)
+    plain.headwise_linear(x, first, stride, weight.float(), out=want, out_first=2, out_head_stride=outputs + 6)
+    got = kernels[dtype].headwise_linear(gpu(x), first, stride, prepared, out=gpu(out), out_first=2, out_head_stride=outputs + 6)
     close(got, want, dtype)
 
 
@@ -128,7 +133,11 @@ def test_join_activate_and_gated_add(kernels, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("tokens,experts,top,hidden,size", [(1, 4, 4, 32, 16), (37, 8, 2, 96, 40), (200, 5, 3, 64, 72)])
+@pytest.mark.parametrize("tokens,experts,top,hidden,size", [
+    (1, 4, 4, 32, 16), (37, 8, 2, 96, 40), (200, 5, 3, 64, 72),
+    # sizes in steps of 32: in bfloat16 the matrix cores, tiles of 16 rows for a few rows an expert and of 64 for many
+    (5, 8, 2, 64, 32), (300, 4, 2, 64, 96), (130, 3, 1, 320, 64),
+])
 def test_routed_experts(kernels, dtype, tokens, experts, top, hidden, size):
     torch.manual_seed(tokens)
     scores = 2 * torch.randn(tokens, experts + 1)
