@@ -1,6 +1,6 @@
-// Operations on rows and on runs of their columns: residual add + layer norm, RMS norm of a run of columns,
-// rotary tables with a magnitude, rotation of a run of columns per head, two streams side by side, an
-// activation, and a gated add.  All arithmetic is float32; inputs and outputs are bfloat16 or float32.
+// Operations on rows and on runs of their columns: RMS norm of a run of columns, rotary tables with a magnitude,
+// rotation of a run of columns per head, two streams side by side, an activation, and a gated add.  All arithmetic
+// is float32; inputs and outputs are bfloat16 or float32.
 #include "common.h"
 
 #define ACT_SILU 0
@@ -15,64 +15,6 @@ __device__ __forceinline__ float activation_of(int activation, float z) {
     case ACT_RELU: return fmaxf(z, 0.f);
     default: return z / (1.f + expf(-z));
   }
-}
-
-// ---------------------------------------------------------------------------- add + layer norm
-// hidden[t] += delta[0][t] + delta[1][t] + ... (if delta); out[t] = (hidden[t] - mean) * rsqrt(var + eps) *
-// weight + bias, var the mean of the squared deviations.  One block per row; a row of up to 8 floats a
-// thread stays in registers between the passes, a longer one is read again.  The sums are added in an order
-// that depends only on the row length.
-#define LN_THREADS 256
-#define LN_KEPT 8
-template <typename TO>
-__global__ __launch_bounds__(LN_THREADS) void add_layer_norm_kernel(float* __restrict__ hidden, const float* __restrict__ delta,
-                                                                    int parts, size_t part_stride, const void* __restrict__ weight,
-                                                                    const void* __restrict__ bias, int weight_is_float,
-                                                                    TO* __restrict__ out, int width, float eps) {
-  __shared__ float shared[17];
-  float* row = hidden + (size_t)blockIdx.x * width;
-  const float* add = delta ? delta + (size_t)blockIdx.x * width : nullptr;
-  float kept[LN_KEPT];
-  float sum = 0.f;
-  int slot = 0;
-  for (int i = threadIdx.x; i < width; i += LN_THREADS, ++slot) {
-    float v = row[i];
-    if (add) {
-      for (int p = 0; p < parts; ++p) v += add[p * part_stride + i];
-      row[i] = v;
-    }
-    if (slot < LN_KEPT) kept[slot] = v;
-    sum += v;
-  }
-  const float mean = block_sum(sum, shared) / (float)width;
-  float squares = 0.f;
-  slot = 0;
-  for (int i = threadIdx.x; i < width; i += LN_THREADS, ++slot) {
-    const float d = (slot < LN_KEPT ? kept[slot] : row[i]) - mean;
-    squares += d * d;
-  }
-  const float scale = rsqrtf(block_sum(squares, shared) / (float)width + eps);
-  TO* dst = out + (size_t)blockIdx.x * width;
-  slot = 0;
-  for (int i = threadIdx.x; i < width; i += LN_THREADS, ++slot) {
-    const float d = (slot < LN_KEPT ? kept[slot] : row[i]) - mean;
-    dst[i] = from_float<TO>(d * scale * load_as_float(weight, weight_is_float, i) + load_as_float(bias, weight_is_float, i));
-  }
-}
-
-extern "C" int llmserve_add_layer_norm(float* hidden, const float* delta, int parts, const void* weight, const void* bias,
-                                       int weight_is_float, void* out, int out_is_float, int rows, int width, float eps,
-                                       hipStream_t stream) {
-  if (rows <= 0) return 0;
-  if (width <= 0 || parts < 1) return ERR_BAD_ARGUMENT;
-  const size_t part_stride = (size_t)rows * width;
-  if (out_is_float)
-    hipLaunchKernelGGL(add_layer_norm_kernel<float>, dim3(rows), dim3(LN_THREADS), 0, stream, hidden, delta, parts, part_stride,
-                       weight, bias, weight_is_float, (float*)out, width, eps);
-  else
-    hipLaunchKernelGGL(add_layer_norm_kernel<bf16_t>, dim3(rows), dim3(LN_THREADS), 0, stream, hidden, delta, parts, part_stride,
-                       weight, bias, weight_is_float, (bf16_t*)out, width, eps);
-  return LAUNCH_STATUS();
 }
 
 // ---------------------------------------------------------------------------- RMS norm of a run of columns

@@ -82,134 +82,188 @@ extern "C" int llmserve_causal_conv(const void* x, int is_float, int tokens, int
 //   q <- q / sqrt(sum q^2 + 1e-6) * dim^-1/2,   k <- k / sqrt(sum k^2 + 1e-6),
 //   beta = sigmoid(b),   g = exp(-exp(rate_h) * softplus(a + step_bias_h)),
 //   S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q            (S [dim, vdim], float32)
-// Column j of S (the state of value dimension j) never meets another column.  A wave owns 16 columns of one (request,
-// head): four neighbouring lanes share a column, each keeping a quarter of its rows (ROWS numbers) in registers for all
-// the tokens of the request's step, and the two sums over a column's rows end with two exchanges between those lanes.
-// The tokens are walked in runs of RUN: first the wave brings the run's q, k, v and controls from memory (all loads
-// under way together: a token by itself would wait for memory every time), makes q and k unit vectors and the decays
-// and betas (lane c those of the run's token c), and leaves them in LDS; then it walks the run token by token out of
-// LDS and registers alone.  The state comes from state[slot, h] ([dim, vdim], columns side by side) and goes back there
-// after the step's last token.
+//
+// Two kernels.  The first is parallel over tokens: it makes q and k unit vectors and the decays and betas, all in
+// float32, and leaves them as the second wants to read them.  The second walks a request's tokens in order.  Column j of
+// S (the state of value dimension j) never meets another column: sixteen neighbouring lanes share a column, each keeping
+// ROWS of its rows in registers for all the tokens of the request's step, and the two sums over a column's rows end with
+// four exchanges between those lanes; a workgroup of four waves owns sixteen columns of one (request, head).  The tokens
+// are walked in runs of RUN: while a run is worked through out of LDS and registers, the next run's k, q, decays, betas
+// and v are on their way from memory into registers (a token by itself would wait for memory every time).  The state is
+// kept as S^T (state[slot, h] is [vdim, dim]: a lane's rows lie side by side) and goes back after the step's last token.
 #define RUN 16
-#define COLUMNS 16
-template <typename T, int ROWS>  // 4 * ROWS >= dim; ROWS a multiple of 4
-__global__ __launch_bounds__(64) void gated_delta_rule_kernel(const T* __restrict__ mixed, const float* __restrict__ controls,
-                                                              const float* __restrict__ rate, const float* __restrict__ step_bias,
-                                                              int heads, int kv_heads, int dim, int vdim,
-                                                              const int* __restrict__ start, const int* __restrict__ slots,
-                                                              float* __restrict__ state, float* __restrict__ out) {
-  constexpr int PADDED = 4 * ROWS, PIECES = (PADDED + WAVE - 1) / WAVE, LINE = 4 * (ROWS + 4);  // (a quarter's rows, then 4 floats: banks)
-  __shared__ __attribute__((aligned(16))) float keys[RUN][LINE], queries[RUN][LINE];
-  __shared__ float decays[RUN], betas[RUN];
-  const int b = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
-  const int column = blockIdx.z * COLUMNS + lane / 4, quarter = lane % 4;
+#define LANES_A_COLUMN 16
+#define COLUMNS 16  // a workgroup's: 256 threads / LANES_A_COLUMN
+
+__host__ __device__ constexpr int delta_rows(int dim) { return 4 * ((dim + 63) / 64); }      // rows a lane keeps
+__host__ __device__ constexpr int delta_line(int rows) { return LANES_A_COLUMN * (rows + 4); }  // a vector in LDS: 4 floats between the lanes' shares (banks)
+
+extern "C" int llmserve_delta_line(int dim) { return delta_line(delta_rows(dim)); }
+
+// unit[t, kv head] = [k | q], each `line` floats: element i of the vector at (i / rows) * (rows + 4) + i % rows, zeros elsewhere.
+// gates[t, head] = (g, beta).  One workgroup a token, a wave a kv head in turn.
+template <typename T>
+__global__ __launch_bounds__(256) void delta_prepare_kernel(const T* __restrict__ mixed, const float* __restrict__ controls,
+                                                            const float* __restrict__ rate, const float* __restrict__ step_bias,
+                                                            int heads, int kv_heads, int dim, int vdim, int rows, int line,
+                                                            float* __restrict__ unit, float* __restrict__ gates) {
+  const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const T* row = mixed + (size_t)t * (2 * kv_heads * dim + heads * vdim);
+  const float q_scale = rsqrtf((float)dim);
+  for (int kv_head = wave; kv_head < kv_heads; kv_head += 4) {
+    float q[4], k[4], q_squares = 0.f, k_squares = 0.f;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int i = p * WAVE + lane;
+      q[p] = i < dim ? to_float(row[kv_head * dim + i]) : 0.f;
+      k[p] = i < dim ? to_float(row[(kv_heads + kv_head) * dim + i]) : 0.f;
+      q_squares += q[p] * q[p];
+      k_squares += k[p] * k[p];
+    }
+    const float q_unit = q_scale / sqrtf(wave_sum(q_squares) + 1e-6f), k_unit = 1.f / sqrtf(wave_sum(k_squares) + 1e-6f);
+    float* dst = unit + ((size_t)t * kv_heads + kv_head) * 2 * line;
+    for (int i = lane; i < 2 * line; i += WAVE) dst[i] = 0.f;  // (the gaps and what lies beyond dim; this wave alone writes here)
+    __builtin_amdgcn_s_waitcnt(0);
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int i = p * WAVE + lane;
+      if (i < dim) {
+        const int where = (i / rows) * (rows + 4) + i % rows;
+        dst[where] = k[p] * k_unit;
+        dst[line + where] = q[p] * q_unit;
+      }
+    }
+  }
+  for (int head = threadIdx.x; head < heads; head += blockDim.x) {
+    const float b_in = controls[(size_t)t * 2 * heads + head], a_in = controls[(size_t)t * 2 * heads + heads + head] + step_bias[head];
+    const float softplus = a_in > 20.f ? a_in : log1pf(expf(a_in));
+    gates[((size_t)t * heads + head) * 2] = expf(-expf(rate[head]) * softplus);
+    gates[((size_t)t * heads + head) * 2 + 1] = 1.f / (1.f + expf(-b_in));
+  }
+}
+
+template <typename T, int ROWS>  // 16 * ROWS >= dim
+__global__ __launch_bounds__(256) void gated_delta_rule_kernel(const T* __restrict__ mixed, const float* __restrict__ unit,
+                                                               const float* __restrict__ gates, int heads, int kv_heads, int dim,
+                                                               int vdim, const int* __restrict__ start, const int* __restrict__ slots,
+                                                               float* __restrict__ state, float* __restrict__ out) {
+  constexpr int LINE = delta_line(ROWS), QUADS = RUN * 2 * LINE / 4, MINE = (QUADS + 255) / 256;  // float4 of a run, and a thread's share
+  __shared__ __attribute__((aligned(16))) float vectors[RUN][2][LINE];
+  __shared__ float decay_beta[RUN][2];
+  const int b = blockIdx.x, head = blockIdx.y, thread = threadIdx.x;
+  const int column = blockIdx.z * COLUMNS + thread / LANES_A_COLUMN, share = thread % LANES_A_COLUMN;
   const bool owns = column < vdim;
   const int first = start[b], last = start[b + 1];
   if (last <= first) return;
   const int kv_head = head / (heads / kv_heads);
   const int row_width = 2 * kv_heads * dim + heads * vdim;
-  float* mine = state + ((size_t)slots[b] * heads + head) * dim * vdim + column;
+  float* mine = state + (((size_t)slots[b] * heads + head) * vdim + column) * dim + share * ROWS;
   float S[ROWS];
 #pragma unroll
-  for (int r = 0; r < ROWS; ++r) {
-    const int i = quarter * ROWS + r;
-    S[r] = (owns && i < dim) ? mine[(size_t)i * vdim] : 0.f;
-  }
-  const float speed = expf(rate[head]), bias = step_bias[head];
-  const float q_scale = rsqrtf((float)dim);
+  for (int r = 0; r < ROWS; ++r) S[r] = (owns && share * ROWS + r < dim) ? mine[r] : 0.f;
+
+  float4 coming[MINE];
+  float v_coming[RUN], gate_coming = 0.f;
+  // asks memory for the run that begins at t0: token c of it is quad / (2 LINE / 4) of the run's quads
+  auto ask = [&](int t0) {
+#pragma unroll
+    for (int j = 0; j < MINE; ++j) {
+      const int quad = thread + j * 256;
+      const int c = quad / (2 * LINE / 4), inside = quad % (2 * LINE / 4);
+      coming[j] = (quad < QUADS && t0 + c < last)
+                      ? ((const float4*)(unit + ((size_t)(t0 + c) * kv_heads + kv_head) * 2 * LINE))[inside]
+                      : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int c = 0; c < RUN; ++c)
+      v_coming[c] = (owns && t0 + c < last) ? to_float(mixed[(size_t)(t0 + c) * row_width + 2 * kv_heads * dim + head * vdim + column]) : 0.f;
+    if (thread < 2 * RUN && t0 + thread / 2 < last) gate_coming = gates[((size_t)(t0 + thread / 2) * heads + head) * 2 + thread % 2];
+  };
+  auto keep = [&]() {
+#pragma unroll
+    for (int j = 0; j < MINE; ++j) {
+      const int quad = thread + j * 256;
+      if (quad < QUADS) ((float4*)&vectors[0][0][0])[quad] = coming[j];
+    }
+    if (thread < 2 * RUN) decay_beta[thread / 2][thread % 2] = gate_coming;
+  };
+
+  ask(first);
+  keep();
+  float v[RUN];
+#pragma unroll
+  for (int c = 0; c < RUN; ++c) v[c] = v_coming[c];
+  __syncthreads();
   for (int t0 = first; t0 < last; t0 += RUN) {
-    float q[RUN][PIECES], k[RUN][PIECES], v[RUN];
-#pragma unroll
-    for (int c = 0; c < RUN; ++c) {
-      const bool valid = t0 + c < last;
-      const T* row = mixed + (size_t)(valid ? t0 + c : t0) * row_width;
-#pragma unroll
-      for (int p = 0; p < PIECES; ++p) {
-        const int i = p * WAVE + lane;
-        q[c][p] = (valid && i < dim) ? to_float(row[kv_head * dim + i]) : 0.f;
-        k[c][p] = (valid && i < dim) ? to_float(row[(kv_heads + kv_head) * dim + i]) : 0.f;
-      }
-      v[c] = (valid && owns) ? to_float(row[2 * kv_heads * dim + head * vdim + column]) : 0.f;
-    }
-    if (lane < RUN && t0 + lane < last) {
-      const size_t at = (size_t)(t0 + lane) * 2 * heads;
-      const float b_in = controls[at + head], a_in = controls[at + heads + head] + bias;
-      const float softplus = a_in > 20.f ? a_in : log1pf(expf(a_in));
-      betas[lane] = 1.f / (1.f + expf(-b_in));
-      decays[lane] = expf(-speed * softplus);
-    }
-#pragma unroll
-    for (int c = 0; c < RUN; ++c) {
-      float q_squares = 0.f, k_squares = 0.f;
-#pragma unroll
-      for (int p = 0; p < PIECES; ++p) {
-        q_squares += q[c][p] * q[c][p];
-        k_squares += k[c][p] * k[c][p];
-      }
-      const float q_unit = q_scale / sqrtf(wave_sum(q_squares) + 1e-6f), k_unit = 1.f / sqrtf(wave_sum(k_squares) + 1e-6f);
-#pragma unroll
-      for (int p = 0; p < PIECES; ++p) {
-        const int i = p * WAVE + lane;
-        if (i < PADDED) {
-          const int where = (i / ROWS) * (ROWS + 4) + i % ROWS;
-          queries[c][where] = q[c][p] * q_unit;
-          keys[c][where] = k[c][p] * k_unit;
-        }
-      }
-    }
-    __syncthreads();
+    const bool more = t0 + RUN < last;
+    if (more) ask(t0 + RUN);
 #pragma unroll
     for (int c = 0; c < RUN; ++c) {
       if (t0 + c < last) {
-        const float g = decays[c], beta = betas[c];
-        const float4* key = (const float4*)&keys[c][quarter * (ROWS + 4)];
-        const float4* query = (const float4*)&queries[c][quarter * (ROWS + 4)];
-        float seen = 0.f;  // (g S)^T k, this lane's rows
+        const float g = decay_beta[c][0], beta = decay_beta[c][1];
+        const float4* key = (const float4*)&vectors[c][0][share * (ROWS + 4)];
+        const float4* query = (const float4*)&vectors[c][1][share * (ROWS + 4)];
+        float seen = 0.f, seen_too = 0.f;  // (g S)^T k over this lane's rows, in two chains
 #pragma unroll
         for (int r = 0; r < ROWS; r += 4) {
           const float4 kk = key[r / 4];
           S[r] *= g; S[r + 1] *= g; S[r + 2] *= g; S[r + 3] *= g;
-          seen += S[r] * kk.x; seen += S[r + 1] * kk.y; seen += S[r + 2] * kk.z; seen += S[r + 3] * kk.w;
+          seen += S[r] * kk.x; seen_too += S[r + 1] * kk.y; seen += S[r + 2] * kk.z; seen_too += S[r + 3] * kk.w;
         }
-        seen += __shfl_xor(seen, 1, WAVE);
-        seen += __shfl_xor(seen, 2, WAVE);
+        seen += seen_too;
+#pragma unroll
+        for (int offset = 1; offset < LANES_A_COLUMN; offset <<= 1) seen += __shfl_xor(seen, offset, WAVE);
         const float u = beta * (v[c] - seen);
-        float read = 0.f;
+        float read = 0.f, read_too = 0.f;
 #pragma unroll
         for (int r = 0; r < ROWS; r += 4) {
           const float4 kk = key[r / 4], qq = query[r / 4];
           S[r] += kk.x * u; S[r + 1] += kk.y * u; S[r + 2] += kk.z * u; S[r + 3] += kk.w * u;
-          read += S[r] * qq.x; read += S[r + 1] * qq.y; read += S[r + 2] * qq.z; read += S[r + 3] * qq.w;
+          read += S[r] * qq.x; read_too += S[r + 1] * qq.y; read += S[r + 2] * qq.z; read_too += S[r + 3] * qq.w;
         }
-        read += __shfl_xor(read, 1, WAVE);
-        read += __shfl_xor(read, 2, WAVE);
-        if (owns && quarter == 0) out[(size_t)(t0 + c) * heads * vdim + head * vdim + column] = read;
+        read += read_too;
+#pragma unroll
+        for (int offset = 1; offset < LANES_A_COLUMN; offset <<= 1) read += __shfl_xor(read, offset, WAVE);
+        if (owns && share == 0) out[(size_t)(t0 + c) * heads * vdim + head * vdim + column] = read;
       }
     }
-    __syncthreads();  // the next run overwrites what this one read
+    __syncthreads();  // everybody has read this run
+    if (more) {
+      keep();
+#pragma unroll
+      for (int c = 0; c < RUN; ++c) v[c] = v_coming[c];
+    }
+    __syncthreads();
   }
   if (owns) {
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-      const int i = quarter * ROWS + r;
-      if (i < dim) mine[(size_t)i * vdim] = S[r];
-    }
+    for (int r = 0; r < ROWS; ++r)
+      if (share * ROWS + r < dim) mine[r] = S[r];
   }
 }
 
+// `unit` has room for tokens * kv_heads * 2 * llmserve_delta_line(dim) floats, `gates` for tokens * heads * 2.
 extern "C" int llmserve_gated_delta_rule(const void* mixed, int is_float, const float* controls, const float* rate,
                                          const float* step_bias, int heads, int kv_heads, int dim, int vdim, const int* start,
-                                         const int* slots, int requests, float* state, float* out, hipStream_t stream) {
-  if (requests <= 0) return 0;
+                                         const int* slots, int requests, int tokens, float* unit, float* gates, float* state,
+                                         float* out, hipStream_t stream) {
+  if (requests <= 0 || tokens <= 0) return 0;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads || dim < 1 || dim > 256 || vdim < 1 || heads > 65535) return ERR_BAD_ARGUMENT;
+  const int rows = delta_rows(dim), line = delta_line(rows);
+  if (is_float)
+    hipLaunchKernelGGL(delta_prepare_kernel<float>, dim3(tokens), dim3(256), 0, stream, (const float*)mixed, controls, rate, step_bias,
+                       heads, kv_heads, dim, vdim, rows, line, unit, gates);
+  else
+    hipLaunchKernelGGL(delta_prepare_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream, (const bf16_t*)mixed, controls, rate,
+                       step_bias, heads, kv_heads, dim, vdim, rows, line, unit, gates);
   const dim3 grid(requests, heads, (vdim + COLUMNS - 1) / COLUMNS);
-#define LAUNCH_RULE(TYPE, ROWS)                                                                                              \
-  hipLaunchKernelGGL((gated_delta_rule_kernel<TYPE, ROWS>), grid, dim3(WAVE), 0, stream, (const TYPE*)mixed, controls, rate, \
-                     step_bias, heads, kv_heads, dim, vdim, start, slots, state, out)
+#define LAUNCH_RULE(TYPE, ROWS)                                                                                                   \
+  hipLaunchKernelGGL((gated_delta_rule_kernel<TYPE, ROWS>), grid, dim3(256), 0, stream, (const TYPE*)mixed, unit, gates, heads, \
+                     kv_heads, dim, vdim, start, slots, state, out)
   if (is_float) {
-    if (dim <= 32) LAUNCH_RULE(float, 8); else if (dim <= 64) LAUNCH_RULE(float, 16); else if (dim <= 128) LAUNCH_RULE(float, 32); else LAUNCH_RULE(float, 64);
+    if (rows == 4) LAUNCH_RULE(float, 4); else if (rows == 8) LAUNCH_RULE(float, 8); else if (rows == 12) LAUNCH_RULE(float, 12); else LAUNCH_RULE(float, 16);
   } else {
-    if (dim <= 32) LAUNCH_RULE(bf16_t, 8); else if (dim <= 64) LAUNCH_RULE(bf16_t, 16); else if (dim <= 128) LAUNCH_RULE(bf16_t, 32); else LAUNCH_RULE(bf16_t, 64);
+    if (rows == 4) LAUNCH_RULE(bf16_t, 4); else if (rows == 8) LAUNCH_RULE(bf16_t, 8); else if (rows == 12) LAUNCH_RULE(bf16_t, 12); else LAUNCH_RULE(bf16_t, 16);
   }
 #undef LAUNCH_RULE
   return LAUNCH_STATUS();

@@ -1,4 +1,4 @@
-// Embedding gather, residual add + RMSNorm, rotary position encoding with the cache
+// Embedding gather, residual add + RMSNorm or layer norm, rotary position encoding with the cache
 // write, SiLU * up, and row gather.  All arithmetic is float32; inputs and outputs are
 // bfloat16 or float32 as the template says.
 #include "common.h"
@@ -194,6 +194,157 @@ extern "C" int llmserve_add_rms_norm(float* hidden, const float* delta, int part
   else
     hipLaunchKernelGGL(add_rms_norm_kernel<bf16_t>, dim3(rows), dim3(threads), 0, stream, hidden, delta, parts,
                        part_stride, weight, weight_is_float, (bf16_t*)out, width, eps);
+  return LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------- add + layer norm
+// hidden[t] += delta[0][t] + delta[1][t] + ... (if delta); out[t] = (hidden[t] - mean) * rsqrt(var + eps) *
+// weight + bias, var the mean of the squared deviations.  One block per row; a row of up to 8 floats a
+// thread stays in registers between the passes, a longer one is read again.  The sums are added in an order
+// that depends only on the row length.
+#define LN_THREADS 256
+#define LN_KEPT 8
+template <typename TO>
+__global__ __launch_bounds__(LN_THREADS) void add_layer_norm_kernel(float* __restrict__ hidden, const float* __restrict__ delta,
+                                                                    int parts, size_t part_stride, const void* __restrict__ weight,
+                                                                    const void* __restrict__ bias, int weight_is_float,
+                                                                    TO* __restrict__ out, int width, float eps) {
+  __shared__ float shared[17];
+  float* row = hidden + (size_t)blockIdx.x * width;
+  const float* add = delta ? delta + (size_t)blockIdx.x * width : nullptr;
+  float kept[LN_KEPT];
+  float sum = 0.f;
+  int slot = 0;
+  for (int i = threadIdx.x; i < width; i += LN_THREADS, ++slot) {
+    float v = row[i];
+    if (add) {
+      for (int p = 0; p < parts; ++p) v += add[p * part_stride + i];
+      row[i] = v;
+    }
+    if (slot < LN_KEPT) kept[slot] = v;
+    sum += v;
+  }
+  const float mean = block_sum(sum, shared) / (float)width;
+  float squares = 0.f;
+  slot = 0;
+  for (int i = threadIdx.x; i < width; i += LN_THREADS, ++slot) {
+    const float d = (slot < LN_KEPT ? kept[slot] : row[i]) - mean;
+    squares += d * d;
+  }
+  const float scale = rsqrtf(block_sum(squares, shared) / (float)width + eps);
+  TO* dst = out + (size_t)blockIdx.x * width;
+  slot = 0;
+  for (int i = threadIdx.x; i < width; i += LN_THREADS, ++slot) {
+    const float d = (slot < LN_KEPT ? kept[slot] : row[i]) - mean;
+    dst[i] = from_float<TO>(d * scale * load_as_float(weight, weight_is_float, i) + load_as_float(bias, weight_is_float, i));
+  }
+}
+
+// The same for rows whose length is a multiple of 4, up to 16,384 floats, as the RMS norm above: the row stays in
+// registers, moves in 16-byte pieces, and all of a thread's loads are on their way before the first is used.
+template <typename TO, int PIECES>
+__global__ __launch_bounds__(1024) void add_layer_norm_vector_kernel(float* __restrict__ hidden, const float* __restrict__ delta,
+                                                                     int parts, size_t part_stride, const void* __restrict__ weight,
+                                                                     const void* __restrict__ bias, int weight_is_float,
+                                                                     TO* __restrict__ out, int width, float eps) {
+  __shared__ float shared[17];
+  const int quads = width / 4;
+  float4* row = (float4*)(hidden + (size_t)blockIdx.x * width);
+  const float* add = delta ? delta + (size_t)blockIdx.x * width : nullptr;
+  float4 v[PIECES], wide[PIECES], wide_bias[PIECES];
+  uint2 narrow[PIECES], narrow_bias[PIECES];
+#pragma unroll
+  for (int j = 0; j < PIECES; ++j) {
+    const int i = min((int)(threadIdx.x + j * blockDim.x), quads - 1);
+    v[j] = row[i];
+    if (weight_is_float) {
+      wide[j] = ((const float4*)weight)[i];
+      wide_bias[j] = ((const float4*)bias)[i];
+    } else {
+      narrow[j] = ((const uint2*)weight)[i];
+      narrow_bias[j] = ((const uint2*)bias)[i];
+    }
+  }
+  if (add) {
+    add_some_parts<PIECES>(v, add, min(parts, 8), part_stride, quads);
+    for (int first = 8; first < parts; first += 8)
+      add_some_parts<PIECES>(v, add + (size_t)first * part_stride, min(parts - first, 8), part_stride, quads);
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < PIECES; ++j) {
+    const int i = threadIdx.x + j * blockDim.x;
+    if (i < quads) {
+      if (add) row[i] = v[j];
+      sum += (v[j].x + v[j].y) + (v[j].z + v[j].w);
+    }
+  }
+  const float mean = block_sum(sum, shared) / (float)width;
+  float squares = 0.f;
+#pragma unroll
+  for (int j = 0; j < PIECES; ++j) {
+    const int i = threadIdx.x + j * blockDim.x;
+    v[j].x -= mean; v[j].y -= mean; v[j].z -= mean; v[j].w -= mean;
+    if (i < quads) squares += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+  }
+  const float scale = rsqrtf(block_sum(squares, shared) / (float)width + eps);
+  TO* dst = out + (size_t)blockIdx.x * width;
+#pragma unroll
+  for (int j = 0; j < PIECES; ++j) {
+    const int i = threadIdx.x + j * blockDim.x;
+    if (i < quads) {
+      float4 w = wide[j], b = wide_bias[j];
+      if (!weight_is_float) {  // a bfloat16 is the upper half of the float32 of the same value
+        w = make_float4(__uint_as_float(narrow[j].x << 16), __uint_as_float(narrow[j].x & 0xffff0000u),
+                        __uint_as_float(narrow[j].y << 16), __uint_as_float(narrow[j].y & 0xffff0000u));
+        b = make_float4(__uint_as_float(narrow_bias[j].x << 16), __uint_as_float(narrow_bias[j].x & 0xffff0000u),
+                        __uint_as_float(narrow_bias[j].y << 16), __uint_as_float(narrow_bias[j].y & 0xffff0000u));
+      }
+      store_four(dst + 4 * i, v[j].x * scale * w.x + b.x, v[j].y * scale * w.y + b.y, v[j].z * scale * w.z + b.z,
+                 v[j].w * scale * w.w + b.w);
+    }
+  }
+}
+
+template <typename TO>
+static void launch_add_layer_norm_vector(float* hidden, const float* delta, int parts, size_t part_stride, const void* weight,
+                                         const void* bias, int weight_is_float, TO* out, int rows, int width, float eps,
+                                         hipStream_t stream) {
+  const int quads = width / 4;
+  const int pieces = quads <= 1024 ? 1 : quads <= 2048 ? 2 : 4;
+  const int threads = ((quads + pieces - 1) / pieces + WAVE - 1) / WAVE * WAVE;
+  if (pieces == 1)
+    hipLaunchKernelGGL((add_layer_norm_vector_kernel<TO, 1>), dim3(rows), dim3(threads), 0, stream, hidden, delta, parts,
+                       part_stride, weight, bias, weight_is_float, out, width, eps);
+  else if (pieces == 2)
+    hipLaunchKernelGGL((add_layer_norm_vector_kernel<TO, 2>), dim3(rows), dim3(threads), 0, stream, hidden, delta, parts,
+                       part_stride, weight, bias, weight_is_float, out, width, eps);
+  else
+    hipLaunchKernelGGL((add_layer_norm_vector_kernel<TO, 4>), dim3(rows), dim3(threads), 0, stream, hidden, delta, parts,
+                       part_stride, weight, bias, weight_is_float, out, width, eps);
+}
+
+extern "C" int llmserve_add_layer_norm(float* hidden, const float* delta, int parts, const void* weight, const void* bias,
+                                       int weight_is_float, void* out, int out_is_float, int rows, int width, float eps,
+                                       hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (width <= 0 || parts < 1) return ERR_BAD_ARGUMENT;
+  const size_t part_stride = (size_t)rows * width;
+  if (width % 4 == 0 && width <= 1024 * 4 * 4) {
+    if (out_is_float)
+      launch_add_layer_norm_vector<float>(hidden, delta, parts, part_stride, weight, bias, weight_is_float, (float*)out, rows,
+                                          width, eps, stream);
+    else
+      launch_add_layer_norm_vector<bf16_t>(hidden, delta, parts, part_stride, weight, bias, weight_is_float, (bf16_t*)out, rows,
+                                           width, eps, stream);
+    return LAUNCH_STATUS();
+  }
+  if (out_is_float)
+    hipLaunchKernelGGL(add_layer_norm_kernel<float>, dim3(rows), dim3(LN_THREADS), 0, stream, hidden, delta, parts, part_stride,
+                       weight, bias, weight_is_float, (float*)out, width, eps);
+  else
+    hipLaunchKernelGGL(add_layer_norm_kernel<bf16_t>, dim3(rows), dim3(LN_THREADS), 0, stream, hidden, delta, parts, part_stride,
+                       weight, bias, weight_is_float, (bf16_t*)out, width, eps);
   return LAUNCH_STATUS();
 }
 

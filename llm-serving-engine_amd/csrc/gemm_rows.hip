@@ -65,7 +65,7 @@ template <int NT, int MT>
 __device__ __forceinline__ void tile_product_mfma(const bf16_t* const (&w_row)[NT], const bf16_t* const (&x_row)[MT], int inner,
                                                   f32x4 (&acc)[NT][MT]) {
   const bf16x8 zero = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll 2
+#pragma unroll(NT * MT <= 2 ? 8 : NT * MT <= 4 ? 4 : 2)
   for (int k0 = 0; k0 < inner; k0 += 32) {
     bf16x8 a[NT], b[MT];
 #pragma unroll
@@ -226,36 +226,53 @@ extern "C" int llmserve_headwise_linear(const void* x, int is_float, int rows, i
 }
 
 // ---------------------------------------------------------------------------- routing
-// One thread a token: s_e = sigmoid(z[t, e]); the `top` experts with the largest s_e + correction_e, the lower index
-// first among equals; chosen[t, i] and weight[t, i] = scale * s_e (no renormalising).
-__global__ void route_kernel(const float* __restrict__ z, int z_stride, int experts, const float* __restrict__ correction,
-                             int top, float scale, int* __restrict__ chosen, float* __restrict__ weight, int tokens) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= tokens) return;
+// One wave a token: s_e = sigmoid(z[t, e]); the `top` experts with the largest s_e + correction_e, the lower index
+// first among equals; chosen[t, i] and weight[t, i] = scale * s_e (no renormalising).  Lane l keeps the experts
+// l, l + 64, ...; a pick is the wave's best of the lanes' best, which is then struck out.
+#define ROUTE_PER_LANE 16
+__global__ __launch_bounds__(WAVE) void route_kernel(const float* __restrict__ z, int z_stride, int experts,
+                                                     const float* __restrict__ correction, int top, float scale,
+                                                     int* __restrict__ chosen, float* __restrict__ weight) {
+  const int t = blockIdx.x, lane = threadIdx.x;
   const float* row = z + (size_t)t * z_stride;
-  int* mine = chosen + (size_t)t * top;
+  float score[ROUTE_PER_LANE], choice[ROUTE_PER_LANE];
+#pragma unroll
+  for (int j = 0; j < ROUTE_PER_LANE; ++j) {
+    const int e = lane + j * WAVE;
+    score[j] = e < experts ? 1.f / (1.f + expf(-row[e])) : 0.f;
+    choice[j] = e < experts ? score[j] + correction[e] : -INFINITY;
+  }
   for (int i = 0; i < top; ++i) {
-    int best = -1;
-    float best_choice = 0.f, best_score = 0.f;
-    for (int e = 0; e < experts; ++e) {
-      bool taken = false;
-      for (int j = 0; j < i; ++j) taken |= mine[j] == e;
-      if (taken) continue;
-      const float score = 1.f / (1.f + expf(-row[e]));
-      const float choice = score + correction[e];
-      if (best < 0 || choice > best_choice) { best = e; best_choice = choice; best_score = score; }
+    float best = -INFINITY, best_score = 0.f;
+    int best_expert = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < ROUTE_PER_LANE; ++j) {
+      const int e = lane + j * WAVE;
+      if (e < experts && (choice[j] > best || best_expert == 0x7fffffff)) { best = choice[j]; best_score = score[j]; best_expert = e; }
     }
-    mine[i] = best;
-    weight[(size_t)t * top + i] = scale * best_score;
+#pragma unroll
+    for (int offset = WAVE / 2; offset > 0; offset >>= 1) {
+      const float other = __shfl_xor(best, offset, WAVE), other_score = __shfl_xor(best_score, offset, WAVE);
+      const int other_expert = __shfl_xor(best_expert, offset, WAVE);
+      if (other_expert != 0x7fffffff && (best_expert == 0x7fffffff || other > best || (other == best && other_expert < best_expert))) {
+        best = other; best_score = other_score; best_expert = other_expert;
+      }
+    }
+    if (lane == 0) {
+      chosen[(size_t)t * top + i] = best_expert;
+      weight[(size_t)t * top + i] = scale * best_score;
+    }
+#pragma unroll
+    for (int j = 0; j < ROUTE_PER_LANE; ++j)
+      if (lane + j * WAVE == best_expert) choice[j] = -INFINITY;
   }
 }
 
 extern "C" int llmserve_route(const float* z, int z_stride, int experts, const float* correction, int top, float scale,
                               int* chosen, float* weight, int tokens, hipStream_t stream) {
   if (tokens <= 0) return 0;
-  if (experts < 1 || top < 1 || top > experts || experts > z_stride) return ERR_BAD_ARGUMENT;
-  hipLaunchKernelGGL(route_kernel, dim3((tokens + 127) / 128), dim3(128), 0, stream, z, z_stride, experts, correction, top,
-                     scale, chosen, weight, tokens);
+  if (experts < 1 || top < 1 || top > experts || experts > z_stride || experts > ROUTE_PER_LANE * WAVE) return ERR_BAD_ARGUMENT;
+  hipLaunchKernelGGL(route_kernel, dim3(tokens), dim3(WAVE), 0, stream, z, z_stride, experts, correction, top, scale, chosen, weight);
   return LAUNCH_STATUS();
 }
 
@@ -356,7 +373,9 @@ extern "C" int llmserve_expert_product(const void* x, int is_float, const int* o
   if (capacity <= 0) return 0;
   if (capacity > 65535 || outputs < 1 || inner < 1) return ERR_BAD_ARGUMENT;
   if (!is_float && inner % 32 == 0) {
-    const int nt = outputs <= 64 ? 1 : outputs <= 128 ? 2 : 4;
+    // a few tiles (decoding) stream their experts' weights: a tile of weight rows a wave, so that many workgroups share the stream
+    int nt = outputs <= 64 ? 1 : outputs <= 128 ? 2 : 4;
+    if (tile_rows == 16 && capacity * ((outputs + 255) / 256) < 1024) nt = 1;
     const dim3 cores((outputs + 64 * nt - 1) / (64 * nt), capacity);
 #define LAUNCH_EXPERTS(NT, MT)                                                                                                  \
   do {                                                                                                                          \

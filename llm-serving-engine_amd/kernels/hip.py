@@ -84,7 +84,8 @@ _SIGNATURES = {
     "llmserve_expert_product": "pipipiipiipiip",
     "llmserve_combine_pairs": "pppipiip",
     "llmserve_causal_conv": "piiiipipppippp",
-    "llmserve_gated_delta_rule": "pipppiiiippippp",
+    "llmserve_gated_delta_rule": "pipppiiiippiippppp",
+    "llmserve_delta_line": "i",
     "llmserve_gated_head_norm": "ppiiipifiiipp",
 }
 _TYPES = {"p": ctypes.c_void_p, "i": ctypes.c_int, "f": ctypes.c_float}
@@ -1063,7 +1064,7 @@ class HipKernels:
             raise KernelError("add_layer_norm: weight and bias are one type and as long as a row")
         out = self._empty((rows, width), self.dtype)
         parts = 1 if delta is None or delta.ndim == 2 else delta.shape[0]
-        status = self._library_of("columns").llmserve_add_layer_norm(
+        status = self._elementwise.llmserve_add_layer_norm(
             _pointer(hidden), _pointer(delta), parts, _pointer(weight), _pointer(bias), _is_float(weight), _pointer(out),
             _is_float(out), rows, width, eps, self._stream,
         )
@@ -1228,12 +1229,17 @@ class HipKernels:
         tokens = mixed.shape[0]
         if mixed.shape[1] != 2 * kv_heads * dim + heads * vdim or controls.shape != (tokens, 2 * heads) or controls.dtype != torch.float32:
             raise KernelError("gated_delta_rule: rows of [q | k | v] and float32 controls [b | a]")
-        if state.dtype != torch.float32 or state.shape[1:] != (heads, dim, vdim) or rate.dtype != torch.float32 or step_bias.dtype != torch.float32:
-            raise KernelError("gated_delta_rule: the state is float32 [slots, heads, dim, vdim]")
+        if state.dtype != torch.float32 or state.shape[1:] != (heads, vdim, dim) or rate.dtype != torch.float32 or step_bias.dtype != torch.float32:
+            raise KernelError("gated_delta_rule: the state is float32 [slots, heads, vdim, dim] (S transposed)")
+        library = self._library_of("delta_rule")
         out = self._empty((tokens, heads * vdim), torch.float32)
-        status = self._library_of("delta_rule").llmserve_gated_delta_rule(
+        line = library.llmserve_delta_line(dim)
+        unit = self._empty((tokens, kv_heads, 2, line), torch.float32)  # unit k and q as the recurrence reads them
+        gates = self._empty((tokens, heads, 2), torch.float32)  # decay and beta
+        status = library.llmserve_gated_delta_rule(
             _pointer(mixed), _is_float(mixed), _pointer(controls), _pointer(rate), _pointer(step_bias), heads, kv_heads, dim, vdim,
-            _pointer(batch.query_start), _pointer(batch.state_slots), batch.state_slots.shape[0], _pointer(state), _pointer(out), self._stream,
+            _pointer(batch.query_start), _pointer(batch.state_slots), batch.state_slots.shape[0], tokens, _pointer(unit), _pointer(gates),
+            _pointer(state), _pointer(out), self._stream,
         )
         _check(status, "gated_delta_rule")
         return out

@@ -39,8 +39,8 @@ class GatedDelta(Mixer):
         S = g S;   u = beta (v - S^T k);   S = S + k u^T;   o = S^T q
 
     then o / rms(o) * norm * silu(W_g x) head by head, and W_o.  Decay, beta, the unit norms and S are
-    float32.  Per request the cache keeps S and the last `taps - 1` inputs of the convolutions, both in
-    state slots that are zero when a request begins."""
+    float32.  Per request the cache keeps S (as S^T, [vdim, dim] a head) and the last `taps - 1` inputs of the
+    convolutions, both in state slots that are zero when a request begins."""
 
     @classmethod
     def tensors(cls, spec: GatedDeltaSpec) -> dict[str, TensorSpec]:
@@ -63,7 +63,7 @@ class GatedDelta(Mixer):
 
     @classmethod
     def cache_need(cls, spec: GatedDeltaSpec) -> dict[str, FixedState]:
-        need = {"state": FixedState((spec.num_heads, spec.dim, spec.vdim))}
+        need = {"state": FixedState((spec.num_heads, spec.vdim, spec.dim))}  # S transposed: a value dimension's column lies side by side
         if spec.taps > 1:
             need["window"] = FixedState((spec.taps - 1, spec.channels))
         return need

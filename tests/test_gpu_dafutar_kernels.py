@@ -185,7 +185,7 @@ def test_gated_delta_rule_over_steps(kernels, dtype, heads, kv_heads, dim, vdim)
     torch.manual_seed(dim)
     plain = TorchKernels(dtype)
     slots = [1, 3]
-    state = torch.zeros(5, heads, dim, vdim)
+    state = torch.zeros(5, heads, vdim, dim)
     on_device = gpu(state)
     rate, bias = torch.randn(heads) - 1.0, torch.randn(heads)
     for counts in ([11, 1], [1, 1], [2, 6]):

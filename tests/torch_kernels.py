@@ -244,7 +244,7 @@ class TorchKernels:
         out = torch.zeros((tokens, heads, vdim))
         row = 0
         for chunk in batch.chunks:
-            S = state[chunk.slot]  # [heads, dim, vdim], updated in place
+            S = state[chunk.slot].transpose(1, 2)  # kept as S^T [heads, vdim, dim]; this view is S [heads, dim, vdim], updated in place
             for t in range(row, row + chunk.count):
                 kt = k[t].repeat_interleave(heads // kv_heads, dim=0)
                 qt = q[t].repeat_interleave(heads // kv_heads, dim=0)
