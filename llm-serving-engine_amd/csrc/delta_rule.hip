@@ -93,6 +93,26 @@ extern "C" int llmserve_causal_conv(const void* x, int is_float, int tokens, int
 // kept as S^T (state[slot, h] is [vdim, dim]: a lane's rows lie side by side) and goes back after the step's last token.
 #define RUN 16
 #define LANES_A_COLUMN 16
+
+// The sum over the sixteen lanes of a row (lanes 16 i .. 16 i + 15), left in every one of them: the lanes are moved by the
+// data-parallel primitives of the vector unit (pairs, pairs of pairs, then the row turned by four and by eight lanes), a
+// few cycles each, where an exchange through the LDS crossbar takes ten times as long; the recurrence waits for two such
+// sums a token.
+__device__ __forceinline__ float moved(float v, int how) {
+  switch (how) {  // (constants: the primitive takes its pattern as an immediate)
+    case 0: return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));   // quad_perm [1, 0, 3, 2]
+    case 1: return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));   // quad_perm [2, 3, 0, 1]
+    case 2: return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xF, 0xF, true));  // row_ror 4
+    default: return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, true)); // row_ror 8
+  }
+}
+__device__ __forceinline__ float row_sum(float v) {
+  v += moved(v, 0);
+  v += moved(v, 1);
+  v += moved(v, 2);
+  v += moved(v, 3);
+  return v;
+}
 #define COLUMNS 16  // a workgroup's: 256 threads / LANES_A_COLUMN
 
 __host__ __device__ constexpr int delta_rows(int dim) { return 4 * ((dim + 63) / 64); }      // rows a lane keeps
@@ -142,14 +162,14 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(const T* __restrict_
   }
 }
 
-template <typename T, int ROWS>  // 16 * ROWS >= dim
+template <typename T, int ROWS, int TOKENS>  // 16 * ROWS >= dim; TOKENS: a run's tokens (RUN, or 2 where every request brings one or two)
 __global__ __launch_bounds__(256) void gated_delta_rule_kernel(const T* __restrict__ mixed, const float* __restrict__ unit,
                                                                const float* __restrict__ gates, int heads, int kv_heads, int dim,
                                                                int vdim, const int* __restrict__ start, const int* __restrict__ slots,
                                                                float* __restrict__ state, float* __restrict__ out) {
-  constexpr int LINE = delta_line(ROWS), QUADS = RUN * 2 * LINE / 4, MINE = (QUADS + 255) / 256;  // float4 of a run, and a thread's share
-  __shared__ __attribute__((aligned(16))) float vectors[RUN][2][LINE];
-  __shared__ float decay_beta[RUN][2];
+  constexpr int LINE = delta_line(ROWS), QUADS = TOKENS * 2 * LINE / 4, MINE = (QUADS + 255) / 256;  // float4 of a run, and a thread's share
+  __shared__ __attribute__((aligned(16))) float vectors[TOKENS][2][LINE];
+  __shared__ float decay_beta[TOKENS][2];
   const int b = blockIdx.x, head = blockIdx.y, thread = threadIdx.x;
   const int column = blockIdx.z * COLUMNS + thread / LANES_A_COLUMN, share = thread % LANES_A_COLUMN;
   const bool owns = column < vdim;
@@ -163,75 +183,92 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(const T* __restri
   for (int r = 0; r < ROWS; ++r) S[r] = (owns && share * ROWS + r < dim) ? mine[r] : 0.f;
 
   float4 coming[MINE];
-  float v_coming[RUN], gate_coming = 0.f;
-  // asks memory for the run that begins at t0: token c of it is quad / (2 LINE / 4) of the run's quads
+  float v_coming[TOKENS], gate_coming = 0.f;
+  // Asks memory for the run that begins at t0: token c of it is quad / (2 LINE / 4) of the run's quads.  The loads stand
+  // in no branch (one would make the wave wait for them at its end): a token beyond the request's last is read from the
+  // last one's place, and `keep` puts zeros for its k and q, a decay of one and a beta of zero instead: walking it changes
+  // nothing, so the walk below has no branches either, and one token's vectors are read before the sums of the token before.
   auto ask = [&](int t0) {
 #pragma unroll
     for (int j = 0; j < MINE; ++j) {
-      const int quad = thread + j * 256;
+      const int quad = min(thread + j * 256, QUADS - 1);
       const int c = quad / (2 * LINE / 4), inside = quad % (2 * LINE / 4);
-      coming[j] = (quad < QUADS && t0 + c < last)
-                      ? ((const float4*)(unit + ((size_t)(t0 + c) * kv_heads + kv_head) * 2 * LINE))[inside]
-                      : make_float4(0.f, 0.f, 0.f, 0.f);
+      coming[j] = ((const float4*)(unit + ((size_t)min(t0 + c, last - 1) * kv_heads + kv_head) * 2 * LINE))[inside];
     }
+    const int my_column = min(column, vdim - 1);
 #pragma unroll
-    for (int c = 0; c < RUN; ++c)
-      v_coming[c] = (owns && t0 + c < last) ? to_float(mixed[(size_t)(t0 + c) * row_width + 2 * kv_heads * dim + head * vdim + column]) : 0.f;
-    if (thread < 2 * RUN && t0 + thread / 2 < last) gate_coming = gates[((size_t)(t0 + thread / 2) * heads + head) * 2 + thread % 2];
+    for (int c = 0; c < TOKENS; ++c)
+      v_coming[c] = to_float(mixed[(size_t)min(t0 + c, last - 1) * row_width + 2 * kv_heads * dim + head * vdim + my_column]);
+    gate_coming = gates[((size_t)min(t0 + (thread / 2) % TOKENS, last - 1) * heads + head) * 2 + thread % 2];
   };
-  auto keep = [&]() {
+  auto keep = [&](int t0) {
 #pragma unroll
     for (int j = 0; j < MINE; ++j) {
       const int quad = thread + j * 256;
-      if (quad < QUADS) ((float4*)&vectors[0][0][0])[quad] = coming[j];
+      const int c = quad / (2 * LINE / 4);
+      if (quad < QUADS) ((float4*)&vectors[0][0][0])[quad] = t0 + c < last ? coming[j] : make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    if (thread < 2 * RUN) decay_beta[thread / 2][thread % 2] = gate_coming;
+    if (thread < 2 * TOKENS) decay_beta[thread / 2][thread % 2] = t0 + thread / 2 < last ? gate_coming : (thread % 2 ? 0.f : 1.f);
   };
 
   ask(first);
-  keep();
-  float v[RUN];
+  keep(first);
+  float v[TOKENS];
 #pragma unroll
-  for (int c = 0; c < RUN; ++c) v[c] = v_coming[c];
+  for (int c = 0; c < TOKENS; ++c) v[c] = v_coming[c];
   __syncthreads();
-  for (int t0 = first; t0 < last; t0 += RUN) {
-    const bool more = t0 + RUN < last;
-    if (more) ask(t0 + RUN);
+  for (int t0 = first; t0 < last; t0 += TOKENS) {
+    const bool more = t0 + TOKENS < last;
+    ask(t0 + TOKENS);  // (beyond the last run: the last token again, dropped)
+    float4 key[ROWS / 4], query[ROWS / 4], next_key[ROWS / 4], next_query[ROWS / 4];
+    float g = decay_beta[0][0], beta = decay_beta[0][1], next_g = 1.f, next_beta = 0.f;
 #pragma unroll
-    for (int c = 0; c < RUN; ++c) {
-      if (t0 + c < last) {
-        const float g = decay_beta[c][0], beta = decay_beta[c][1];
-        const float4* key = (const float4*)&vectors[c][0][share * (ROWS + 4)];
-        const float4* query = (const float4*)&vectors[c][1][share * (ROWS + 4)];
-        float seen = 0.f, seen_too = 0.f;  // (g S)^T k over this lane's rows, in two chains
+    for (int r = 0; r < ROWS / 4; ++r) {
+      key[r] = ((const float4*)&vectors[0][0][share * (ROWS + 4)])[r];
+      query[r] = ((const float4*)&vectors[0][1][share * (ROWS + 4)])[r];
+    }
 #pragma unroll
-        for (int r = 0; r < ROWS; r += 4) {
-          const float4 kk = key[r / 4];
-          S[r] *= g; S[r + 1] *= g; S[r + 2] *= g; S[r + 3] *= g;
-          seen += S[r] * kk.x; seen_too += S[r + 1] * kk.y; seen += S[r + 2] * kk.z; seen_too += S[r + 3] * kk.w;
+    for (int c = 0; c < TOKENS; ++c) {
+      if (c + 1 < TOKENS) {
+        next_g = decay_beta[c + 1][0];
+        next_beta = decay_beta[c + 1][1];
+#pragma unroll
+        for (int r = 0; r < ROWS / 4; ++r) {
+          next_key[r] = ((const float4*)&vectors[c + 1][0][share * (ROWS + 4)])[r];
+          next_query[r] = ((const float4*)&vectors[c + 1][1][share * (ROWS + 4)])[r];
         }
-        seen += seen_too;
+      }
+      float seen = 0.f, seen_too = 0.f;  // (g S)^T k over this lane's rows, in two chains
 #pragma unroll
-        for (int offset = 1; offset < LANES_A_COLUMN; offset <<= 1) seen += __shfl_xor(seen, offset, WAVE);
-        const float u = beta * (v[c] - seen);
-        float read = 0.f, read_too = 0.f;
+      for (int r = 0; r < ROWS; r += 4) {
+        const float4 kk = key[r / 4];
+        S[r] *= g; S[r + 1] *= g; S[r + 2] *= g; S[r + 3] *= g;
+        seen += S[r] * kk.x; seen_too += S[r + 1] * kk.y; seen += S[r + 2] * kk.z; seen_too += S[r + 3] * kk.w;
+      }
+      seen = row_sum(seen + seen_too);
+      const float u = beta * (v[c] - seen);
+      float read = 0.f, read_too = 0.f;
 #pragma unroll
-        for (int r = 0; r < ROWS; r += 4) {
-          const float4 kk = key[r / 4], qq = query[r / 4];
-          S[r] += kk.x * u; S[r + 1] += kk.y * u; S[r + 2] += kk.z * u; S[r + 3] += kk.w * u;
-          read += S[r] * qq.x; read_too += S[r + 1] * qq.y; read += S[r + 2] * qq.z; read_too += S[r + 3] * qq.w;
-        }
-        read += read_too;
+      for (int r = 0; r < ROWS; r += 4) {
+        const float4 kk = key[r / 4], qq = query[r / 4];
+        S[r] += kk.x * u; S[r + 1] += kk.y * u; S[r + 2] += kk.z * u; S[r + 3] += kk.w * u;
+        read += S[r] * qq.x; read_too += S[r + 1] * qq.y; read += S[r + 2] * qq.z; read_too += S[r + 3] * qq.w;
+      }
+      read = row_sum(read + read_too);
+      if (owns && share == 0 && t0 + c < last) out[(size_t)(t0 + c) * heads * vdim + head * vdim + column] = read;
+      g = next_g;
+      beta = next_beta;
 #pragma unroll
-        for (int offset = 1; offset < LANES_A_COLUMN; offset <<= 1) read += __shfl_xor(read, offset, WAVE);
-        if (owns && share == 0) out[(size_t)(t0 + c) * heads * vdim + head * vdim + column] = read;
+      for (int r = 0; r < ROWS / 4; ++r) {
+        key[r] = next_key[r];
+        query[r] = next_query[r];
       }
     }
     __syncthreads();  // everybody has read this run
     if (more) {
-      keep();
+      keep(t0 + TOKENS);
 #pragma unroll
-      for (int c = 0; c < RUN; ++c) v[c] = v_coming[c];
+      for (int c = 0; c < TOKENS; ++c) v[c] = v_coming[c];
     }
     __syncthreads();
   }
@@ -245,8 +282,8 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(const T* __restri
 // `unit` has room for tokens * kv_heads * 2 * llmserve_delta_line(dim) floats, `gates` for tokens * heads * 2.
 extern "C" int llmserve_gated_delta_rule(const void* mixed, int is_float, const float* controls, const float* rate,
                                          const float* step_bias, int heads, int kv_heads, int dim, int vdim, const int* start,
-                                         const int* slots, int requests, int tokens, float* unit, float* gates, float* state,
-                                         float* out, hipStream_t stream) {
+                                         const int* slots, int requests, int tokens, int longest, float* unit, float* gates,
+                                         float* state, float* out, hipStream_t stream) {
   if (requests <= 0 || tokens <= 0) return 0;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads || dim < 1 || dim > 256 || vdim < 1 || heads > 65535) return ERR_BAD_ARGUMENT;
   const int rows = delta_rows(dim), line = delta_line(rows);
@@ -257,9 +294,16 @@ extern "C" int llmserve_gated_delta_rule(const void* mixed, int is_float, const 
     hipLaunchKernelGGL(delta_prepare_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream, (const bf16_t*)mixed, controls, rate,
                        step_bias, heads, kv_heads, dim, vdim, rows, line, unit, gates);
   const dim3 grid(requests, heads, (vdim + COLUMNS - 1) / COLUMNS);
-#define LAUNCH_RULE(TYPE, ROWS)                                                                                                   \
-  hipLaunchKernelGGL((gated_delta_rule_kernel<TYPE, ROWS>), grid, dim3(256), 0, stream, (const TYPE*)mixed, unit, gates, heads, \
-                     kv_heads, dim, vdim, start, slots, state, out)
+  // `longest`: the most tokens a request brings; one or two (decoding) are walked in runs of two
+#define LAUNCH_RULE(TYPE, ROWS)                                                                                                          \
+  do {                                                                                                                                   \
+    if (longest <= 2)                                                                                                                    \
+      hipLaunchKernelGGL((gated_delta_rule_kernel<TYPE, ROWS, 2>), grid, dim3(256), 0, stream, (const TYPE*)mixed, unit, gates, heads,   \
+                         kv_heads, dim, vdim, start, slots, state, out);                                                                 \
+    else                                                                                                                                 \
+      hipLaunchKernelGGL((gated_delta_rule_kernel<TYPE, ROWS, RUN>), grid, dim3(256), 0, stream, (const TYPE*)mixed, unit, gates, heads, \
+                         kv_heads, dim, vdim, start, slots, state, out);                                                                 \
+  } while (0)
   if (is_float) {
     if (rows == 4) LAUNCH_RULE(float, 4); else if (rows == 8) LAUNCH_RULE(float, 8); else if (rows == 12) LAUNCH_RULE(float, 12); else LAUNCH_RULE(float, 16);
   } else {

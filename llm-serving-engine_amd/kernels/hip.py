@@ -84,7 +84,7 @@ _SIGNATURES = {
     "llmserve_expert_product": "pipipiipiipiip",
     "llmserve_combine_pairs": "pppipiip",
     "llmserve_causal_conv": "piiiipipppippp",
-    "llmserve_gated_delta_rule": "pipppiiiippiippppp",
+    "llmserve_gated_delta_rule": "pipppiiiippiiippppp",
     "llmserve_delta_line": "i",
     "llmserve_gated_head_norm": "ppiiipifiiipp",
 }
@@ -1238,7 +1238,8 @@ class HipKernels:
         gates = self._empty((tokens, heads, 2), torch.float32)  # decay and beta
         status = library.llmserve_gated_delta_rule(
             _pointer(mixed), _is_float(mixed), _pointer(controls), _pointer(rate), _pointer(step_bias), heads, kv_heads, dim, vdim,
-            _pointer(batch.query_start), _pointer(batch.state_slots), batch.state_slots.shape[0], tokens, _pointer(unit), _pointer(gates),
+            _pointer(batch.query_start), _pointer(batch.state_slots), batch.state_slots.shape[0], tokens, int(getattr(batch, "max_query_length", tokens)),
+            _pointer(unit), _pointer(gates),
             _pointer(state), _pointer(out), self._stream,
         )
         _check(status, "gated_delta_rule")
