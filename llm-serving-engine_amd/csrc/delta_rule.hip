@@ -162,11 +162,76 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(const T* __restrict_
   }
 }
 
+// The same with the convolutions in front: the token's row of x is [q | k | v | ...] before the convolutions, `channels`
+// of them; the workgroup convolves them (as causal_conv_kernel does), keeps the results in LDS as float32, and goes on
+// as above; the convolved v goes to values[t] (float32 [heads * vdim]).  The window is read here and written by the
+// recurrence kernel, which runs behind this one.
+template <typename T>
+__global__ __launch_bounds__(256) void delta_prepare_conv_kernel(const T* __restrict__ x, int x_stride, int channels,
+                                                                 const float* __restrict__ taps, int width,
+                                                                 const int* __restrict__ token_request, const int* __restrict__ start,
+                                                                 const int* __restrict__ slots, const float* __restrict__ window,
+                                                                 const float* __restrict__ controls, const float* __restrict__ rate,
+                                                                 const float* __restrict__ step_bias, int heads, int kv_heads, int dim,
+                                                                 int vdim, int rows, int line, float* __restrict__ unit,
+                                                                 float* __restrict__ gates, float* __restrict__ values) {
+  extern __shared__ float convolved[];  // [channels]
+  const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int b = token_request[t], i0 = t - start[b];
+  const float* kept = window ? window + (size_t)slots[b] * (width - 1) * channels : nullptr;
+  for (int c = threadIdx.x; c < channels; c += blockDim.x) {
+    float sum = 0.f;
+    for (int j = 0; j < width; ++j) {
+      const int n = i0 - (width - 1) + j;
+      const float v = n >= 0 ? to_float(x[(size_t)(t - i0 + n) * x_stride + c]) : kept[(size_t)(width - 1 + n) * channels + c];
+      sum += taps[(size_t)c * width + j] * v;
+    }
+    const float y = sum / (1.f + expf(-sum));
+    convolved[c] = y;
+    if (c >= 2 * kv_heads * dim) values[(size_t)t * heads * vdim + c - 2 * kv_heads * dim] = y;
+  }
+  __syncthreads();
+  const float q_scale = rsqrtf((float)dim);
+  for (int kv_head = wave; kv_head < kv_heads; kv_head += 4) {
+    float q[4], k[4], q_squares = 0.f, k_squares = 0.f;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int i = p * WAVE + lane;
+      q[p] = i < dim ? convolved[kv_head * dim + i] : 0.f;
+      k[p] = i < dim ? convolved[(kv_heads + kv_head) * dim + i] : 0.f;
+      q_squares += q[p] * q[p];
+      k_squares += k[p] * k[p];
+    }
+    const float q_unit = q_scale / sqrtf(wave_sum(q_squares) + 1e-6f), k_unit = 1.f / sqrtf(wave_sum(k_squares) + 1e-6f);
+    float* dst = unit + ((size_t)t * kv_heads + kv_head) * 2 * line;
+    for (int i = lane; i < 2 * line; i += WAVE) dst[i] = 0.f;
+    __builtin_amdgcn_s_waitcnt(0);
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int i = p * WAVE + lane;
+      if (i < dim) {
+        const int where = (i / rows) * (rows + 4) + i % rows;
+        dst[where] = k[p] * k_unit;
+        dst[line + where] = q[p] * q_unit;
+      }
+    }
+  }
+  for (int head = threadIdx.x; head < heads; head += blockDim.x) {
+    const float b_in = controls[(size_t)t * 2 * heads + head], a_in = controls[(size_t)t * 2 * heads + heads + head] + step_bias[head];
+    const float softplus = a_in > 20.f ? a_in : log1pf(expf(a_in));
+    gates[((size_t)t * heads + head) * 2] = expf(-expf(rate[head]) * softplus);
+    gates[((size_t)t * heads + head) * 2 + 1] = 1.f / (1.f + expf(-b_in));
+  }
+}
+
 template <typename T, int ROWS, int TOKENS>  // 16 * ROWS >= dim; TOKENS: a run's tokens (RUN, or 2 where every request brings one or two)
-__global__ __launch_bounds__(256) void gated_delta_rule_kernel(const T* __restrict__ mixed, const float* __restrict__ unit,
-                                                               const float* __restrict__ gates, int heads, int kv_heads, int dim,
-                                                               int vdim, const int* __restrict__ start, const int* __restrict__ slots,
-                                                               float* __restrict__ state, float* __restrict__ out) {
+__global__ __launch_bounds__(256) void gated_delta_rule_kernel(const T* __restrict__ mixed, const float* __restrict__ values,
+                                                               const float* __restrict__ unit, const float* __restrict__ gates,
+                                                               int heads, int kv_heads, int dim, int vdim,
+                                                               const int* __restrict__ start, const int* __restrict__ slots,
+                                                               float* __restrict__ state, float* __restrict__ out,
+                                                               const T* __restrict__ x, int x_stride, int channels, int width,
+                                                               float* __restrict__ window) {
   constexpr int LINE = delta_line(ROWS), QUADS = TOKENS * 2 * LINE / 4, MINE = (QUADS + 255) / 256;  // float4 of a run, and a thread's share
   __shared__ __attribute__((aligned(16))) float vectors[TOKENS][2][LINE];
   __shared__ float decay_beta[TOKENS][2];
@@ -175,6 +240,25 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(const T* __restri
   const bool owns = column < vdim;
   const int first = start[b], last = start[b + 1];
   if (last <= first) return;
+  if (window && head == 0 && blockIdx.z == 0) {
+    // With the convolutions in the kernel before this one (`values` given): the request's kept inputs move on, as
+    // conv_window_kernel does it; every thread reads what it needs of a channel before it writes.
+    float* kept = window + (size_t)slots[b] * (width - 1) * channels;
+    const int count = last - first;
+    for (int c = thread; c < channels; c += 256) {
+      float next[MAX_TAPS];
+#pragma unroll
+      for (int i = 0; i < MAX_TAPS; ++i) {
+        if (i < width - 1) {
+          const int n = count - (width - 1) + i;
+          next[i] = n >= 0 ? to_float(x[(size_t)(first + n) * x_stride + c]) : kept[(size_t)(i + count) * channels + c];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < MAX_TAPS; ++i)
+        if (i < width - 1) kept[(size_t)i * channels + c] = next[i];
+    }
+  }
   const int kv_head = head / (heads / kv_heads);
   const int row_width = 2 * kv_heads * dim + heads * vdim;
   float* mine = state + (((size_t)slots[b] * heads + head) * vdim + column) * dim + share * ROWS;
@@ -198,7 +282,8 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(const T* __restri
     const int my_column = min(column, vdim - 1);
 #pragma unroll
     for (int c = 0; c < TOKENS; ++c)
-      v_coming[c] = to_float(mixed[(size_t)min(t0 + c, last - 1) * row_width + 2 * kv_heads * dim + head * vdim + my_column]);
+      v_coming[c] = values ? values[(size_t)min(t0 + c, last - 1) * heads * vdim + head * vdim + my_column]
+                           : to_float(mixed[(size_t)min(t0 + c, last - 1) * row_width + 2 * kv_heads * dim + head * vdim + my_column]);
     gate_coming = gates[((size_t)min(t0 + (thread / 2) % TOKENS, last - 1) * heads + head) * 2 + thread % 2];
   };
   auto keep = [&](int t0) {
@@ -280,6 +365,27 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(const T* __restri
 }
 
 // `unit` has room for tokens * kv_heads * 2 * llmserve_delta_line(dim) floats, `gates` for tokens * heads * 2.
+// `longest`: the most tokens a request brings; one or two (decoding) are walked in runs of two.
+template <typename T>
+static int launch_rule(const T* mixed, const float* values, const float* unit, const float* gates, int heads, int kv_heads, int dim,
+                       int vdim, const int* start, const int* slots, int requests, int longest, float* state, float* out, const T* x,
+                       int x_stride, int channels, int width, float* window, hipStream_t stream) {
+  const dim3 grid(requests, heads, (vdim + COLUMNS - 1) / COLUMNS);
+  const int rows = delta_rows(dim);
+#define LAUNCH_RULE(ROWS)                                                                                                         \
+  do {                                                                                                                            \
+    if (longest <= 2)                                                                                                             \
+      hipLaunchKernelGGL((gated_delta_rule_kernel<T, ROWS, 2>), grid, dim3(256), 0, stream, mixed, values, unit, gates, heads,    \
+                         kv_heads, dim, vdim, start, slots, state, out, x, x_stride, channels, width, window);                    \
+    else                                                                                                                          \
+      hipLaunchKernelGGL((gated_delta_rule_kernel<T, ROWS, RUN>), grid, dim3(256), 0, stream, mixed, values, unit, gates, heads,  \
+                         kv_heads, dim, vdim, start, slots, state, out, x, x_stride, channels, width, window);                    \
+  } while (0)
+  if (rows == 4) LAUNCH_RULE(4); else if (rows == 8) LAUNCH_RULE(8); else if (rows == 12) LAUNCH_RULE(12); else LAUNCH_RULE(16);
+#undef LAUNCH_RULE
+  return LAUNCH_STATUS();
+}
+
 extern "C" int llmserve_gated_delta_rule(const void* mixed, int is_float, const float* controls, const float* rate,
                                          const float* step_bias, int heads, int kv_heads, int dim, int vdim, const int* start,
                                          const int* slots, int requests, int tokens, int longest, float* unit, float* gates,
@@ -287,30 +393,44 @@ extern "C" int llmserve_gated_delta_rule(const void* mixed, int is_float, const 
   if (requests <= 0 || tokens <= 0) return 0;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads || dim < 1 || dim > 256 || vdim < 1 || heads > 65535) return ERR_BAD_ARGUMENT;
   const int rows = delta_rows(dim), line = delta_line(rows);
-  if (is_float)
+  if (is_float) {
     hipLaunchKernelGGL(delta_prepare_kernel<float>, dim3(tokens), dim3(256), 0, stream, (const float*)mixed, controls, rate, step_bias,
                        heads, kv_heads, dim, vdim, rows, line, unit, gates);
-  else
-    hipLaunchKernelGGL(delta_prepare_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream, (const bf16_t*)mixed, controls, rate,
-                       step_bias, heads, kv_heads, dim, vdim, rows, line, unit, gates);
-  const dim3 grid(requests, heads, (vdim + COLUMNS - 1) / COLUMNS);
-  // `longest`: the most tokens a request brings; one or two (decoding) are walked in runs of two
-#define LAUNCH_RULE(TYPE, ROWS)                                                                                                          \
-  do {                                                                                                                                   \
-    if (longest <= 2)                                                                                                                    \
-      hipLaunchKernelGGL((gated_delta_rule_kernel<TYPE, ROWS, 2>), grid, dim3(256), 0, stream, (const TYPE*)mixed, unit, gates, heads,   \
-                         kv_heads, dim, vdim, start, slots, state, out);                                                                 \
-    else                                                                                                                                 \
-      hipLaunchKernelGGL((gated_delta_rule_kernel<TYPE, ROWS, RUN>), grid, dim3(256), 0, stream, (const TYPE*)mixed, unit, gates, heads, \
-                         kv_heads, dim, vdim, start, slots, state, out);                                                                 \
-  } while (0)
-  if (is_float) {
-    if (rows == 4) LAUNCH_RULE(float, 4); else if (rows == 8) LAUNCH_RULE(float, 8); else if (rows == 12) LAUNCH_RULE(float, 12); else LAUNCH_RULE(float, 16);
-  } else {
-    if (rows == 4) LAUNCH_RULE(bf16_t, 4); else if (rows == 8) LAUNCH_RULE(bf16_t, 8); else if (rows == 12) LAUNCH_RULE(bf16_t, 12); else LAUNCH_RULE(bf16_t, 16);
+    return launch_rule<float>((const float*)mixed, nullptr, unit, gates, heads, kv_heads, dim, vdim, start, slots, requests, longest,
+                              state, out, nullptr, 0, 0, 0, nullptr, stream);
   }
-#undef LAUNCH_RULE
-  return LAUNCH_STATUS();
+  hipLaunchKernelGGL(delta_prepare_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream, (const bf16_t*)mixed, controls, rate,
+                     step_bias, heads, kv_heads, dim, vdim, rows, line, unit, gates);
+  return launch_rule<bf16_t>((const bf16_t*)mixed, nullptr, unit, gates, heads, kv_heads, dim, vdim, start, slots, requests, longest,
+                             state, out, nullptr, 0, 0, 0, nullptr, stream);
+}
+
+// Convolutions, unit vectors, gates and the recurrence in two kernels: x [tokens, x_stride] holds [q | k | v] before the
+// convolutions in its first `channels` columns; `values` has room for tokens * heads * vdim floats.
+extern "C" int llmserve_conv_gated_delta_rule(const void* x, int is_float, int x_stride, int channels, const float* taps, int width,
+                                              const int* token_request, float* window, const float* controls, const float* rate,
+                                              const float* step_bias, int heads, int kv_heads, int dim, int vdim, const int* start,
+                                              const int* slots, int requests, int tokens, int longest, float* unit, float* gates,
+                                              float* values, float* state, float* out, hipStream_t stream) {
+  if (requests <= 0 || tokens <= 0) return 0;
+  if (heads < 1 || kv_heads < 1 || heads % kv_heads || dim < 1 || dim > 256 || vdim < 1 || heads > 65535) return ERR_BAD_ARGUMENT;
+  if (width < 1 || width > MAX_TAPS || channels != 2 * kv_heads * dim + heads * vdim || channels > x_stride || channels > 12288 ||
+      (width > 1 && !window))
+    return ERR_BAD_ARGUMENT;
+  const int rows = delta_rows(dim), line = delta_line(rows);
+  const size_t lds = (size_t)channels * sizeof(float);
+  if (is_float) {
+    hipLaunchKernelGGL(delta_prepare_conv_kernel<float>, dim3(tokens), dim3(256), lds, stream, (const float*)x, x_stride, channels, taps,
+                       width, token_request, start, slots, (const float*)window, controls, rate, step_bias, heads, kv_heads, dim, vdim,
+                       rows, line, unit, gates, values);
+    return launch_rule<float>(nullptr, values, unit, gates, heads, kv_heads, dim, vdim, start, slots, requests, longest, state, out,
+                              (const float*)x, x_stride, channels, width, width > 1 ? window : nullptr, stream);
+  }
+  hipLaunchKernelGGL(delta_prepare_conv_kernel<bf16_t>, dim3(tokens), dim3(256), lds, stream, (const bf16_t*)x, x_stride, channels,
+                     taps, width, token_request, start, slots, (const float*)window, controls, rate, step_bias, heads, kv_heads, dim,
+                     vdim, rows, line, unit, gates, values);
+  return launch_rule<bf16_t>(nullptr, values, unit, gates, heads, kv_heads, dim, vdim, start, slots, requests, longest, state, out,
+                             (const bf16_t*)x, x_stride, channels, width, width > 1 ? window : nullptr, stream);
 }
 
 // ---------------------------------------------------------------------------- gated norm of the read-out

@@ -168,6 +168,49 @@ __global__ __launch_bounds__(256) void expert_product_mfma_kernel(const bf16_t* 
   }
 }
 
+// The experts' products of a step of few rows (decoding): every tile holds a few rows of one expert, and the product is a
+// stream of that expert's weights.  A workgroup owns 16 weight rows of one tile's expert and its four waves take the
+// 32-wide steps of K in turn (wave v the steps v, v + 4, ...), so that four times as many loads are under way as with a
+// wave a tile of weight rows; the waves' partial tiles are added through LDS in wave order.
+template <typename TO>
+__global__ __launch_bounds__(256) void expert_stream_kernel(const bf16_t* __restrict__ x, const int* __restrict__ order, int top,
+                                                            const bf16_t* __restrict__ w, int outputs, int inner,
+                                                            const int* __restrict__ tiles, TO* __restrict__ out, int activation) {
+  __shared__ f32x4 partial[4][WAVE];
+  const int* tile = tiles + 3 * (size_t)blockIdx.y;
+  const int expert = tile[0], first = tile[1], rows = tile[2];
+  if (rows == 0) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+  const int n = min((int)blockIdx.x * 16 + r, outputs - 1);
+  const bf16_t* w_row = w + ((size_t)expert * outputs + n) * inner + g * 8;
+  const bf16_t* x_row = nullptr;
+  if (r < rows) {
+    const int place = first + r;
+    x_row = x + (size_t)(top > 0 ? order[place] / top : place) * inner + g * 8;
+  }
+  const bf16x8 zero = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+  f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
+  const int steps = inner / 32;
+#pragma unroll 4
+  for (int step = wave; step < steps; step += 4) {
+    const bf16x8 a = *(const bf16x8*)(w_row + step * 32);
+    const bf16x8 b = x_row ? *(const bf16x8*)(x_row + step * 32) : zero;
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+  }
+  partial[wave][lane] = acc;
+  __syncthreads();
+  if (wave != 0 || r >= rows) return;
+  f32x4 total = partial[0][lane];
+#pragma unroll
+  for (int v = 1; v < 4; ++v) total += partial[v][lane];
+  TO* dst = out + (size_t)(first + r) * outputs;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int column = blockIdx.x * 16 + g * 4 + i;
+    if (column < outputs) dst[column] = from_float<TO>(activation_of(activation, total[i]));
+  }
+}
+
 // ---------------------------------------------------------------------------- a product per head
 // out[t, out_first + h * out_head_stride + n] = sum_k x[t, first + h * head_stride + k] * w[h, n, k]
 template <typename T>
@@ -374,8 +417,18 @@ extern "C" int llmserve_expert_product(const void* x, int is_float, const int* o
   if (capacity > 65535 || outputs < 1 || inner < 1) return ERR_BAD_ARGUMENT;
   if (!is_float && inner % 32 == 0) {
     // a few tiles (decoding) stream their experts' weights: a tile of weight rows a wave, so that many workgroups share the stream
-    int nt = outputs <= 64 ? 1 : outputs <= 128 ? 2 : 4;
-    if (tile_rows == 16 && capacity * ((outputs + 255) / 256) < 1024) nt = 1;
+    if (tile_rows == 16 && capacity * ((outputs + 15) / 16) <= 8192) {
+      // a few tiles (decoding) stream their experts' weights: sixteen weight rows a workgroup, K dealt out to its waves
+      const dim3 streams((outputs + 15) / 16, capacity);
+      if (out_is_float)
+        hipLaunchKernelGGL(expert_stream_kernel<float>, streams, dim3(256), 0, stream, (const bf16_t*)x, order, top, (const bf16_t*)w,
+                           outputs, inner, tiles, (float*)out, activation);
+      else
+        hipLaunchKernelGGL(expert_stream_kernel<bf16_t>, streams, dim3(256), 0, stream, (const bf16_t*)x, order, top, (const bf16_t*)w,
+                           outputs, inner, tiles, (bf16_t*)out, activation);
+      return LAUNCH_STATUS();
+    }
+    const int nt = outputs <= 64 ? 1 : outputs <= 128 ? 2 : 4;
     const dim3 cores((outputs + 64 * nt - 1) / (64 * nt), capacity);
 #define LAUNCH_EXPERTS(NT, MT)                                                                                                  \
   do {                                                                                                                          \
@@ -413,20 +466,27 @@ extern "C" int llmserve_expert_product(const void* x, int is_float, const int* o
 }
 
 // ---------------------------------------------------------------------------- the tokens' weighted sums
-// out[t] = sum_i weight[t, i] * rows[place[t * top + i]], in the order of i.
+// out[t] = sum_i weight[t, i] * rows[place[t * top + i]], in the order of i; with `shared`, plus
+// sigmoid(gates[t, gate_column]) * shared[t] (an expert that every token uses, behind a gate of its own).
 __global__ void combine_pairs_kernel(const float* __restrict__ rows, const int* __restrict__ place, const float* __restrict__ weight,
-                                     int top, float* __restrict__ out, int width) {
+                                     int top, float* __restrict__ out, int width, const float* __restrict__ shared,
+                                     const float* __restrict__ gates, int gate_stride, int gate_column) {
   const int t = blockIdx.x;
+  const float gate = shared ? 1.f / (1.f + expf(-gates[(size_t)t * gate_stride + gate_column])) : 0.f;
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
     float sum = 0.f;
     for (int i = 0; i < top; ++i) sum += weight[(size_t)t * top + i] * rows[(size_t)place[(size_t)t * top + i] * width + c];
+    if (shared) sum += gate * shared[(size_t)t * width + c];
     out[(size_t)t * width + c] = sum;
   }
 }
 
 extern "C" int llmserve_combine_pairs(const float* rows, const int* place, const float* weight, int top, float* out, int tokens,
-                                      int width, hipStream_t stream) {
+                                      int width, const float* shared, const float* gates, int gate_stride, int gate_column,
+                                      hipStream_t stream) {
   if (tokens <= 0) return 0;
-  hipLaunchKernelGGL(combine_pairs_kernel, dim3(tokens), dim3(256), 0, stream, rows, place, weight, top, out, width);
+  if (shared && (!gates || gate_column < 0 || gate_column >= gate_stride)) return ERR_BAD_ARGUMENT;
+  hipLaunchKernelGGL(combine_pairs_kernel, dim3(tokens), dim3(256), 0, stream, rows, place, weight, top, out, width, shared, gates,
+                     gate_stride, gate_column);
   return LAUNCH_STATUS();
 }

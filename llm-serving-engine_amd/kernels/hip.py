@@ -82,7 +82,8 @@ _SIGNATURES = {
     "llmserve_route": "piipifppip",
     "llmserve_sort_pairs": "piipppiip",
     "llmserve_expert_product": "pipipiipiipiip",
-    "llmserve_combine_pairs": "pppipiip",
+    "llmserve_combine_pairs": "pppipiippiip",
+    "llmserve_conv_gated_delta_rule": "piiipipppppiiiippiiipppppp",
     "llmserve_causal_conv": "piiiipipppippp",
     "llmserve_gated_delta_rule": "pipppiiiippiiippppp",
     "llmserve_delta_line": "i",
@@ -1174,10 +1175,11 @@ class HipKernels:
             raise KernelError(f"experts: no kernel applies the activation {activation!r} (known: {', '.join(_ACTIVATIONS)})")
         return torch.stack(list(ups)).contiguous(), torch.stack(list(downs)).contiguous(), activation
 
-    def expert_feed_forward(self, x, experts, chosen, weights) -> torch.Tensor:
+    def expert_feed_forward(self, x, experts, chosen, weights, shared=None, gates=None, gate_column: int = 0) -> torch.Tensor:
         """sum over a token's chosen experts of weight * down(act(up x)), float32 [T, hidden].  The (token, choice)
         pairs are sorted by expert on the device, the two products run over tiles of one expert's rows, and a last
-        kernel adds each token's rows up in the order of its choices."""
+        kernel adds each token's rows up in the order of its choices; with `shared` (float32 [T, hidden]) it adds
+        sigmoid(gates[:, gate_column]) * shared as well."""
         ups, downs, activation = experts
         tokens, top = chosen.shape
         count, size, hidden = ups.shape
@@ -1201,8 +1203,12 @@ class HipKernels:
         _check(library.llmserve_expert_product(
             _pointer(inner), _is_float(inner), _pointer(order), 0, _pointer(downs), hidden, size, _pointer(tiles), capacity, tile_rows, _pointer(rows),
             1, -1, self._stream), "experts: second product")
+        if shared is not None and (shared.dtype != torch.float32 or shared.shape != (tokens, hidden) or gates is None or gates.dtype != torch.float32):
+            raise KernelError("experts: the shared rows and their gates are float32")
         out = self._empty((tokens, hidden), torch.float32)
-        _check(library.llmserve_combine_pairs(_pointer(rows), _pointer(place), _pointer(weights), top, _pointer(out), tokens, hidden, self._stream), "experts: sum")
+        _check(library.llmserve_combine_pairs(
+            _pointer(rows), _pointer(place), _pointer(weights), top, _pointer(out), tokens, hidden, _pointer(shared),
+            _pointer(gates if shared is not None else None), gates.shape[1] if shared is not None else 1, gate_column, self._stream), "experts: sum")
         return out
 
     # ------------------------------------------------------------------ the gated delta rule
@@ -1243,6 +1249,38 @@ class HipKernels:
             _pointer(state), _pointer(out), self._stream,
         )
         _check(status, "gated_delta_rule")
+        return out
+
+    def conv_gated_delta_rule(self, projected, channels: int, taps, activation: str, controls, rate, step_bias, heads: int, kv_heads: int,
+                              dim: int, vdim: int, batch, window, state) -> torch.Tensor:
+        """`causal_conv` and `gated_delta_rule` in two kernels: one, parallel over tokens, convolves, makes the unit vectors
+        and the gates; the other walks the tokens and moves the kept inputs on.  What lies between stays float32."""
+        if activation != "silu":
+            raise KernelError(f"causal_conv: no kernel applies {activation!r} behind the convolution")
+        tokens, width = projected.shape[0], taps.shape[1]
+        if channels > 12288:  # (more than the first kernel keeps in LDS)
+            mixed = self.causal_conv(projected, channels, taps, activation, batch, window)
+            return self.gated_delta_rule(mixed, controls, rate, step_bias, heads, kv_heads, dim, vdim, batch, state)
+        if channels != 2 * kv_heads * dim + heads * vdim or taps.dtype != torch.float32 or taps.shape[0] != channels:
+            raise KernelError("conv_gated_delta_rule: the convolutions run over [q | k | v], float32 taps a channel")
+        if width > 1 and (window is None or window.dtype != torch.float32 or window.shape[1:] != (width - 1, channels)):
+            raise KernelError("conv_gated_delta_rule: the kept inputs are float32 [slots, taps - 1, channels]")
+        if controls.shape != (tokens, 2 * heads) or controls.dtype != torch.float32 or state.dtype != torch.float32 or state.shape[1:] != (heads, vdim, dim):
+            raise KernelError("conv_gated_delta_rule: float32 controls [b | a] and a float32 state [slots, heads, vdim, dim]")
+        library = self._library_of("delta_rule")
+        out = self._empty((tokens, heads * vdim), torch.float32)
+        line = library.llmserve_delta_line(dim)
+        unit = self._empty((tokens, kv_heads, 2, line), torch.float32)
+        gates = self._empty((tokens, heads, 2), torch.float32)
+        values = self._empty((tokens, heads * vdim), torch.float32)
+        status = library.llmserve_conv_gated_delta_rule(
+            _pointer(projected), _is_float(projected), projected.shape[1], channels, _pointer(taps), width, _pointer(batch.token_sequence),
+            _pointer(window if width > 1 else None), _pointer(controls), _pointer(rate), _pointer(step_bias), heads, kv_heads, dim, vdim,
+            _pointer(batch.query_start), _pointer(batch.state_slots), batch.state_slots.shape[0], tokens,
+            int(getattr(batch, "max_query_length", tokens)), _pointer(unit), _pointer(gates), _pointer(values), _pointer(state), _pointer(out),
+            self._stream,
+        )
+        _check(status, "conv_gated_delta_rule")
         return out
 
     def gated_head_norm(self, read, gates, gate_first: int, weight, eps: float, heads: int, vdim: int, activation: str) -> torch.Tensor:

@@ -86,9 +86,10 @@ class GatedDelta(Mixer):
         projected = kernels.linear(x, self.inputs)  # [T, q | k | v | g]
         controls = kernels.linear(x, self.controls, out_dtype=torch.float32)  # [T, b | a]
         window = cell["window"].state if "window" in cell else None
-        mixed = kernels.causal_conv(projected, spec.channels, self.taps, "silu", batch, window)  # [T, q | k | v]
-        read = kernels.gated_delta_rule(
-            mixed, controls, self.rate, self.step_bias, spec.num_heads, spec.num_kv_heads, spec.dim, spec.vdim, batch, cell["state"].state
+        # the convolutions over [q | k | v], their silu, the unit vectors, the gates and the recurrence
+        read = kernels.conv_gated_delta_rule(
+            projected, spec.channels, self.taps, "silu", controls, self.rate, self.step_bias, spec.num_heads, spec.num_kv_heads,
+            spec.dim, spec.vdim, batch, window, cell["state"].state,
         )  # float32 [T, heads * vdim]
         gated = kernels.gated_head_norm(read, projected, spec.channels, self.norm, spec.eps, spec.num_heads, spec.vdim, "silu")
         return kernels.linear(gated, self.out, out_dtype=torch.float32, partial=True)

@@ -68,9 +68,9 @@ class RoutedExperts(FeedForward):
         kernels, spec = self.kernels, self.spec
         scores = kernels.linear(x, self.router, out_dtype=torch.float32)  # [T, experts (+ 1)]
         chosen, weights = kernels.route(scores, spec.num_experts, self.correction, spec.top, spec.route_scale, spec.scoring)
-        routed = kernels.expert_feed_forward(x, self.experts, chosen, weights)  # float32 [T, hidden]
         if self.shared_up is None:
-            return routed
+            return kernels.expert_feed_forward(x, self.experts, chosen, weights)  # float32 [T, hidden]
         inner = kernels.activate(kernels.linear(x, self.shared_up), spec.shared_activation)
         shared = kernels.linear(inner, self.shared_down, out_dtype=torch.float32)
-        return kernels.add_gated_rows(routed, shared, scores, spec.num_experts, "sigmoid")
+        # the kernel that adds a token's experts up adds the gated shared expert too
+        return kernels.expert_feed_forward(x, self.experts, chosen, weights, shared=shared, gates=scores, gate_column=spec.num_experts)

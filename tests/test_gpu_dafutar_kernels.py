@@ -156,6 +156,10 @@ def test_routed_experts(kernels, dtype, tokens, experts, top, hidden, size):
     close(got, want, dtype)
     again = kernels[dtype].expert_feed_forward(gpu(x), prepared, chosen, weights)
     assert torch.equal(got, again)  # whatever order the sort gave the rows of an expert
+    shared = torch.randn(tokens, hidden)
+    want = plain.expert_feed_forward(x, plain.prepare_experts(ups, downs, "gelu"), want_chosen, want_weights, shared=shared, gates=scores, gate_column=experts)
+    got = kernels[dtype].expert_feed_forward(gpu(x), prepared, chosen, weights, shared=gpu(shared), gates=gpu(scores), gate_column=experts)
+    close(got, want, dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -211,3 +215,32 @@ def test_gated_head_norm(kernels, dtype, heads, vdim):
     want = TorchKernels(dtype).gated_head_norm(read, gates, 5, weight, 1e-5, heads, vdim, "silu")
     got = kernels[dtype].gated_head_norm(gpu(read), gpu(gates), 5, gpu(weight), 1e-5, heads, vdim, "silu")
     close(got, want, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,dim,vdim,taps", [(6, 3, 64, 64, 4), (2, 2, 16, 96, 1), (4, 1, 80, 32, 3), (3, 3, 130, 70, 2)])
+def test_convolutions_and_delta_rule_in_one(kernels, dtype, heads, kv_heads, dim, vdim, taps):
+    """The fused form against the two operations one after the other, over steps of many tokens, of one and of two."""
+    torch.manual_seed(dim + taps)
+    plain = TorchKernels(torch.float32)  # (the fused form keeps what lies between the two in float32)
+    channels = 2 * kv_heads * dim + heads * vdim
+    weights = torch.randn(channels, taps) / taps**0.5
+    slots = [1, 3]
+    state, window = torch.zeros(5, heads, vdim, dim), (torch.zeros(5, taps - 1, channels) if taps > 1 else None)
+    on_device, window_on_device = gpu(state), (gpu(window) if window is not None else None)
+    rate, bias = torch.randn(heads) - 1.0, torch.randn(heads)
+    for counts in ([37, 1], [1, 1], [2, 1], [2, 19]):
+        tokens = sum(counts)
+        projected = torch.randn(tokens, channels + 11).to(dtype)
+        controls = 2 * torch.randn(tokens, 2 * heads)
+        host, device = step_of(counts, [0, 0], slots, "cpu"), step_of(counts, [0, 0], slots, "cuda")
+        device.max_query_length = max(counts)
+        want = plain.conv_gated_delta_rule(projected.float(), channels, weights, "silu", controls, rate, bias, heads, kv_heads, dim, vdim, host, window, state)
+        got = kernels[dtype].conv_gated_delta_rule(
+            gpu(projected), channels, gpu(weights), "silu", gpu(controls), gpu(rate), gpu(bias), heads, kv_heads, dim, vdim, device,
+            window_on_device, on_device,
+        )
+        close(got, want, torch.float32, atol=3e-4, rtol=3e-4)
+        close(on_device, state, torch.float32, atol=3e-4, rtol=3e-4)
+        if window is not None:
+            close(window_on_device, window, torch.float32, atol=0, rtol=0)

@@ -275,7 +275,11 @@ class TorchKernels:
     def prepare_experts(self, ups, downs, activation):
         return (torch.stack([w.float() for w in ups]), torch.stack([w.float() for w in downs]), activation)
 
-    def expert_feed_forward(self, x, experts, chosen, weights):
+    def conv_gated_delta_rule(self, projected, channels, taps, activation, controls, rate, step_bias, heads, kv_heads, dim, vdim, batch, window, state):
+        mixed = self.causal_conv(projected, channels, taps, activation, batch, window)
+        return self.gated_delta_rule(mixed, controls, rate, step_bias, heads, kv_heads, dim, vdim, batch, state)
+
+    def expert_feed_forward(self, x, experts, chosen, weights, shared=None, gates=None, gate_column=0):
         ups, downs, activation = experts
         out = torch.zeros((x.shape[0], downs.shape[1]))
         for t in range(x.shape[0]):
@@ -283,4 +287,6 @@ class TorchKernels:
                 e = int(chosen[t, slot])
                 inner = self.activate((x[t].float() @ ups[e].T).to(self.dtype), activation).float()
                 out[t] += weights[t, slot] * (inner @ downs[e].T)
+        if shared is not None:
+            out += torch.sigmoid(gates[:, gate_column : gate_column + 1].float()) * shared
         return out
