@@ -162,12 +162,41 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(const T* __restrict_
   }
 }
 
+// One channel's convolution at token number i0 of its request, silu applied.  WIDTH > 0: the taps are known when the
+// kernel is compiled and all their loads are asked for together; WIDTH 0: any number of taps, one after the other.
+template <typename T, int WIDTH>
+__device__ __forceinline__ float convolved_channel(const T* __restrict__ x, int x_stride, int channels, const float* __restrict__ taps,
+                                                   int width, const float* __restrict__ kept, int t, int i0, int c) {
+  float sum = 0.f;
+  if (WIDTH > 0) {
+    float v[WIDTH > 0 ? WIDTH : 1], w[WIDTH > 0 ? WIDTH : 1];
+#pragma unroll
+    for (int j = 0; j < WIDTH; ++j) {
+      const int n = i0 - (WIDTH - 1) + j;
+      // (both addresses are valid whichever is meant: no load stands in a branch)
+      const float fresh = to_float(x[(size_t)(t - i0 + max(n, 0)) * x_stride + c]);
+      const float old = WIDTH > 1 ? kept[(size_t)min(WIDTH - 1 + n, WIDTH - 2) * channels + c] : 0.f;
+      v[j] = n >= 0 ? fresh : old;
+      w[j] = taps[(size_t)c * WIDTH + j];
+    }
+#pragma unroll
+    for (int j = 0; j < WIDTH; ++j) sum += w[j] * v[j];
+  } else {
+    for (int j = 0; j < width; ++j) {
+      const int n = i0 - (width - 1) + j;
+      const float v = n >= 0 ? to_float(x[(size_t)(t - i0 + n) * x_stride + c]) : kept[(size_t)(width - 1 + n) * channels + c];
+      sum += taps[(size_t)c * width + j] * v;
+    }
+  }
+  return sum / (1.f + expf(-sum));
+}
+
 // The same with the convolutions in front: the token's row of x is [q | k | v | ...] before the convolutions, `channels`
 // of them; the workgroup convolves them (as causal_conv_kernel does), keeps the results in LDS as float32, and goes on
 // as above; the convolved v goes to values[t] (float32 [heads * vdim]).  The window is read here and written by the
 // recurrence kernel, which runs behind this one.
-template <typename T>
-__global__ __launch_bounds__(256) void delta_prepare_conv_kernel(const T* __restrict__ x, int x_stride, int channels,
+template <typename T, int WIDTH>
+__global__ __launch_bounds__(1024) void delta_prepare_conv_kernel(const T* __restrict__ x, int x_stride, int channels,
                                                                  const float* __restrict__ taps, int width,
                                                                  const int* __restrict__ token_request, const int* __restrict__ start,
                                                                  const int* __restrict__ slots, const float* __restrict__ window,
@@ -180,19 +209,13 @@ __global__ __launch_bounds__(256) void delta_prepare_conv_kernel(const T* __rest
   const int b = token_request[t], i0 = t - start[b];
   const float* kept = window ? window + (size_t)slots[b] * (width - 1) * channels : nullptr;
   for (int c = threadIdx.x; c < channels; c += blockDim.x) {
-    float sum = 0.f;
-    for (int j = 0; j < width; ++j) {
-      const int n = i0 - (width - 1) + j;
-      const float v = n >= 0 ? to_float(x[(size_t)(t - i0 + n) * x_stride + c]) : kept[(size_t)(width - 1 + n) * channels + c];
-      sum += taps[(size_t)c * width + j] * v;
-    }
-    const float y = sum / (1.f + expf(-sum));
+    const float y = convolved_channel<T, WIDTH>(x, x_stride, channels, taps, width, kept, t, i0, c);
     convolved[c] = y;
     if (c >= 2 * kv_heads * dim) values[(size_t)t * heads * vdim + c - 2 * kv_heads * dim] = y;
   }
   __syncthreads();
   const float q_scale = rsqrtf((float)dim);
-  for (int kv_head = wave; kv_head < kv_heads; kv_head += 4) {
+  for (int kv_head = wave; kv_head < kv_heads; kv_head += blockDim.x / WAVE) {
     float q[4], k[4], q_squares = 0.f, k_squares = 0.f;
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
@@ -240,12 +263,13 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(const T* __restri
   const bool owns = column < vdim;
   const int first = start[b], last = start[b + 1];
   if (last <= first) return;
-  if (window && head == 0 && blockIdx.z == 0) {
+  if (window) {
     // With the convolutions in the kernel before this one (`values` given): the request's kept inputs move on, as
-    // conv_window_kernel does it; every thread reads what it needs of a channel before it writes.
+    // conv_window_kernel does it, the channels dealt out to the request's workgroups; every thread reads what it needs
+    // of a channel before it writes.
     float* kept = window + (size_t)slots[b] * (width - 1) * channels;
     const int count = last - first;
-    for (int c = thread; c < channels; c += 256) {
+    for (int c = (head * gridDim.z + blockIdx.z) * 256 + thread; c < channels; c += gridDim.y * gridDim.z * 256) {
       float next[MAX_TAPS];
 #pragma unroll
       for (int i = 0; i < MAX_TAPS; ++i) {
@@ -419,16 +443,27 @@ extern "C" int llmserve_conv_gated_delta_rule(const void* x, int is_float, int x
     return ERR_BAD_ARGUMENT;
   const int rows = delta_rows(dim), line = delta_line(rows);
   const size_t lds = (size_t)channels * sizeof(float);
+  const int threads = channels > 512 ? 1024 : 256;
+#define LAUNCH_PREPARE(TYPE, WIDTH)                                                                                                  \
+  hipLaunchKernelGGL((delta_prepare_conv_kernel<TYPE, WIDTH>), dim3(tokens), dim3(threads), lds, stream, (const TYPE*)x, x_stride,    \
+                     channels, taps, width, token_request, start, slots, (const float*)window, controls, rate, step_bias, heads,     \
+                     kv_heads, dim, vdim, rows, line, unit, gates, values)
+#define LAUNCH_PREPARE_BY_WIDTH(TYPE)                                                                                       \
+  switch (width) {                                                                                                          \
+    case 1: LAUNCH_PREPARE(TYPE, 1); break;                                                                                 \
+    case 2: LAUNCH_PREPARE(TYPE, 2); break;                                                                                 \
+    case 3: LAUNCH_PREPARE(TYPE, 3); break;                                                                                 \
+    case 4: LAUNCH_PREPARE(TYPE, 4); break;                                                                                 \
+    default: LAUNCH_PREPARE(TYPE, 0); break;                                                                                \
+  }
   if (is_float) {
-    hipLaunchKernelGGL(delta_prepare_conv_kernel<float>, dim3(tokens), dim3(256), lds, stream, (const float*)x, x_stride, channels, taps,
-                       width, token_request, start, slots, (const float*)window, controls, rate, step_bias, heads, kv_heads, dim, vdim,
-                       rows, line, unit, gates, values);
+    LAUNCH_PREPARE_BY_WIDTH(float)
     return launch_rule<float>(nullptr, values, unit, gates, heads, kv_heads, dim, vdim, start, slots, requests, longest, state, out,
                               (const float*)x, x_stride, channels, width, width > 1 ? window : nullptr, stream);
   }
-  hipLaunchKernelGGL(delta_prepare_conv_kernel<bf16_t>, dim3(tokens), dim3(256), lds, stream, (const bf16_t*)x, x_stride, channels,
-                     taps, width, token_request, start, slots, (const float*)window, controls, rate, step_bias, heads, kv_heads, dim,
-                     vdim, rows, line, unit, gates, values);
+  LAUNCH_PREPARE_BY_WIDTH(bf16_t)
+#undef LAUNCH_PREPARE_BY_WIDTH
+#undef LAUNCH_PREPARE
   return launch_rule<bf16_t>(nullptr, values, unit, gates, heads, kv_heads, dim, vdim, start, slots, requests, longest, state, out,
                              (const bf16_t*)x, x_stride, channels, width, width > 1 ? window : nullptr, stream);
 }
