@@ -12,7 +12,7 @@
 #include "common.h"
 
 #define KEYS_PER_TILE 128
-#define MAX_DIM 512
+#define MAX_DIM 1024
 
 template <typename T>
 __global__ __launch_bounds__(KEYS_PER_TILE) void attention_generic_kernel(

@@ -65,7 +65,7 @@ template <int NT, int MT>
 __device__ __forceinline__ void tile_product_mfma(const bf16_t* const (&w_row)[NT], const bf16_t* const (&x_row)[MT], int inner,
                                                   f32x4 (&acc)[NT][MT]) {
   const bf16x8 zero = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll(NT * MT <= 2 ? 8 : NT * MT <= 4 ? 4 : 2)
+#pragma unroll(NT * MT <= 2 ? 8 : 4)
   for (int k0 = 0; k0 < inner; k0 += 32) {
     bf16x8 a[NT], b[MT];
 #pragma unroll

@@ -72,6 +72,95 @@ class Kernels(Protocol):
         `prepare_linear` returned), followed by `linear(that, project, float32, partial=True)`, whose result
         is returned instead (a library may let that product finish what the attention left undone)."""
 
+    # ------------------------------------------------------------------ layer norm, runs of columns, products per head
+
+    def add_layer_norm(
+        self, hidden: torch.Tensor, delta: torch.Tensor | None, weight: torch.Tensor, bias: torch.Tensor, eps: float
+    ) -> torch.Tensor:
+        """`hidden += delta` in place (float32), then (rows - mean) * rsqrt(var + eps) * weight + bias in the run dtype."""
+
+    def new_rows(self, rows: int, width: int) -> torch.Tensor:
+        """An uninitialised [rows, width] tensor in the run dtype for operations that write runs of its columns."""
+
+    def rms_norm_columns(
+        self, x: torch.Tensor, first: int, weight: torch.Tensor, eps: float, out: torch.Tensor | None = None,
+        out_first: int = 0, copies: int = 1, copy_stride: int = 0,
+    ) -> torch.Tensor:
+        """RMS norm (float32) of the columns [first, first + len(weight)) of x's rows, times weight; written to a new
+        tensor, or to `copies` places of `out`'s rows, `copy_stride` columns apart, from column `out_first`."""
+
+    def rotary_table(self, batch: Any, frequencies: torch.Tensor, magnitude: float = 1.0) -> torch.Tensor:
+        """float32 [T, len(frequencies), 2]: magnitude * (cos, sin) of position * frequency for the step's tokens."""
+
+    def rotate_columns(
+        self, x: torch.Tensor, first: int, head_stride: int, heads: int, width: int, table: torch.Tensor, dims: int,
+        out: torch.Tensor, out_first: int, out_head_stride: int,
+    ) -> torch.Tensor:
+        """For every head h: `width` columns of x from first + h * head_stride to out from out_first + h *
+        out_head_stride; the first `dims` of them rotated in adjacent pairs by the token's table row, the rest copied."""
+
+    def prepare_headwise_linear(self, weight: torch.Tensor) -> Any:
+        """[heads, N, K] weights in whatever layout `headwise_linear` wants."""
+
+    def headwise_linear(
+        self, x: torch.Tensor, first: int, head_stride: int, weights: Any, out: torch.Tensor | None = None,
+        out_first: int = 0, out_head_stride: int | None = None,
+    ) -> torch.Tensor:
+        """For every head h: x[:, first + h * head_stride : + K] @ W_h^T -> out[:, out_first + h * out_head_stride : + N]
+        (a new [T, heads * N] tensor if `out` is None), run dtype, float32 sums."""
+
+    def join_rows(self, hidden: torch.Tensor, delta: torch.Tensor | None, embedded: torch.Tensor) -> torch.Tensor:
+        """[hidden + delta | embedded] in the run dtype, [T, 2 hidden]."""
+
+    def activate(self, x: torch.Tensor, activation: str) -> torch.Tensor:
+        """act(x) elementwise (silu, gelu, gelu_tanh, relu), in x's type."""
+
+    def add_gated_rows(self, target: torch.Tensor, rows: torch.Tensor, gates: torch.Tensor, column: int, squash: str) -> torch.Tensor:
+        """target += squash(gates[:, column]) * rows, float32, in place."""
+
+    # ------------------------------------------------------------------ the gated delta rule
+
+    def causal_conv(self, x: torch.Tensor, channels: int, taps: torch.Tensor, activation: str, batch: Any, window: torch.Tensor | None) -> torch.Tensor:
+        """act of the causal convolution per channel over each request's tokens, of the first `channels` columns of x;
+        taps float32 [channels, width], the last column the current token's.  `window` float32 [slots, width - 1,
+        channels] holds each request's last inputs (zeros at its start) and is moved on."""
+
+    def gated_delta_rule(
+        self, mixed: torch.Tensor, controls: torch.Tensor, rate: torch.Tensor, step_bias: torch.Tensor, heads: int,
+        kv_heads: int, dim: int, vdim: int, batch: Any, state: torch.Tensor,
+    ) -> torch.Tensor:
+        """mixed [T, q | k | v], controls float32 [T, b | a]; q, k to unit length (q times dim^-1/2), beta = sigmoid(b),
+        g = exp(-exp(rate) softplus(a + step_bias)); per request and head, token by token: S = g S; u = beta (v - S^T k);
+        S += k u^T; o = S^T q.  `state` float32 [slots, heads, vdim, dim] holds S^T and is updated.  -> float32 [T, heads * vdim]."""
+
+    def conv_gated_delta_rule(
+        self, projected: torch.Tensor, channels: int, taps: torch.Tensor, activation: str, controls: torch.Tensor,
+        rate: torch.Tensor, step_bias: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, batch: Any,
+        window: torch.Tensor | None, state: torch.Tensor,
+    ) -> torch.Tensor:
+        """`causal_conv` followed by `gated_delta_rule` (a library may fuse them and keep what lies between in float32)."""
+
+    def gated_head_norm(
+        self, read: torch.Tensor, gates: torch.Tensor, gate_first: int, weight: torch.Tensor, eps: float, heads: int,
+        vdim: int, activation: str,
+    ) -> torch.Tensor:
+        """Per head: read / rms(read) * weight * act(gates[:, gate_first + h * vdim : + vdim]) -> run dtype [T, heads * vdim]."""
+
+    # ------------------------------------------------------------------ routed experts
+
+    def route(self, scores: torch.Tensor, experts: int, correction: torch.Tensor, top: int, scale: float, scoring: str):
+        """s = squash(scores[:, :experts]); the `top` largest of s + correction choose (the lower index among equals);
+        -> (int32 [T, top] experts, float32 [T, top] weights = scale * s of the chosen)."""
+
+    def prepare_experts(self, ups: list[torch.Tensor], downs: list[torch.Tensor], activation: str) -> Any: ...
+
+    def expert_feed_forward(
+        self, x: torch.Tensor, experts: Any, chosen: torch.Tensor, weights: torch.Tensor, shared: torch.Tensor | None = None,
+        gates: torch.Tensor | None = None, gate_column: int = 0,
+    ) -> torch.Tensor:
+        """sum over a token's chosen experts of weight * down_e(act(up_e x)) (+ sigmoid(gates[:, gate_column]) * shared),
+        float32 [T, hidden]; the inner rows are rounded to the run dtype between the two products."""
+
     def gather_rows(self, hidden: torch.Tensor, delta: torch.Tensor | None, rows: torch.Tensor) -> torch.Tensor:
         """float32 (hidden + delta)[rows]."""
 

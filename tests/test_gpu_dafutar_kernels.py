@@ -45,7 +45,7 @@ def step_of(counts, starts, slots, device):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("width", [24, 320, 2500])
+@pytest.mark.parametrize("width", [24, 30, 320, 1001, 2500])
 def test_add_layer_norm(kernels, dtype, width):
     torch.manual_seed(width)
     hidden, delta = torch.randn(5, width) + 0.5, 0.3 * torch.randn(3, 5, width)
