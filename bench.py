@@ -24,6 +24,11 @@ prints the reference's own kernel-level table instead (one attention layer, cont
 times the paged attention of prompt portions alone (the configuration's heads; whole prompts of 2,048
 and 8,192 tokens, a 2,048-token portion behind 8,192 to 32,704 keys, sixteen prompts of 512) and prints
 microseconds and PFLOP/s, counting the causal half only.
+
+    python bench.py --op dafutar
+
+measures the engine's second architecture (configs/dafutar-w1536.json, configs/dafutar-w3584.json) beside a Qwen2 of the
+same width, number of layer runs and vocabulary: decoding at --batch and the prefill of --prefill-len tokens.
 """
 
 from __future__ import annotations

@@ -291,3 +291,27 @@ def test_greedy_generation_through_the_engine(mixed_folder):
     core = EngineCore(runner, SchedulerConfig(max_batch_size=3, max_tokens_per_step=24), prefill_chunk_size=8)
     assert core.generate(prompts, GenerationConfig(max_new_tokens=7)) == expected
     assert runner.cache.used_pages == 0
+
+
+ONE_KIND = {
+    "only the delta rule": cases.config_of([(cases.delta(), cases.moe(4, 2, 1.0, 8, 8)), (cases.delta(heads=2, kv_heads=1, dim=8, vdim=24, conv=2), None)], loop=(0, 1, 2)),
+    "only latent attention": cases.config_of([(cases.latent(), cases.dense(24)), (cases.latent(heads=2, dim=8, rot_dim=4, vdim=8, kv_rank=12), None)]),
+}
+
+
+@pytest.mark.parametrize("name", list(ONE_KIND))
+def test_models_of_one_kind_of_layer_through_the_scheduler(tmp_path, name):
+    """A model that keeps no pages at all, and one that keeps no state: steps, and generation through the scheduler."""
+    folder = cases.write_folder(tmp_path / "m", ONE_KIND[name], seed=5)
+    config, tensors = plain.read_folder(folder)
+    prompts = [cases.tokens_of(n, 61, seed=60 + n) for n in (3, 11, 20)]
+    expected = []
+    for prompt in prompts:
+        tokens = list(prompt)
+        for _ in range(5):
+            tokens.append(int(torch.argmax(plain.forward(config, tensors, tokens)[0][-1])))
+        expected.append(tokens[len(prompt):])
+    runner = runner_for(folder, page=4, pages=32, slots=3)
+    core = EngineCore(runner, SchedulerConfig(max_batch_size=2, max_tokens_per_step=16), prefill_chunk_size=6)
+    assert core.generate(prompts, GenerationConfig(max_new_tokens=5)) == expected
+    assert len(runner.cache.sequences) == 0

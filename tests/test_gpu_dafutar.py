@@ -12,7 +12,7 @@ from llmserve_amd.weights import load_model_folder
 from tests import dafutar_cases as cases
 from tests.gpu_helpers import TraceBuilder, replay
 from tests.plain import dafutar_plain as plain
-from tests.test_dafutar import PLACES, far_key_case
+from tests.test_dafutar import ONE_KIND, PLACES, far_key_case
 
 pytestmark = pytest.mark.gpu
 
@@ -36,7 +36,7 @@ def folders(tmp_path_factory):
     # sizes the matrix-core kernels take (rows of 64 + 32, heads of 64) beside the odd ones of the other two
     wide = cases.config_of(
         [
-            (cases.delta(heads=4, kv_heads=2, dim=64, vdim=128, conv=4), cases.moe(8, 2, 1.5, 64, 96)),
+            (cases.delta(heads=4, kv_heads=2, dim=64, vdim=128, conv=4), cases.moe(8, 3, 1.25, 64, 128)),
             (cases.latent(heads=4, dim=32, rot_dim=32, vdim=48, q_rank=96, kv_rank=64), cases.dense(256)),
         ],
         loop=(0, 2, 2), vocab=300, width=128,
@@ -164,6 +164,25 @@ def test_greedy_generation_through_the_engine(folders, kernels):
     core = EngineCore(runner, SchedulerConfig(max_batch_size=3, max_tokens_per_step=24), prefill_chunk_size=8)
     assert core.generate(prompts, GenerationConfig(max_new_tokens=12)) == expected
     assert runner.cache.used_pages == 0
+    runner.close()
+
+
+@pytest.mark.parametrize("name", list(ONE_KIND))
+def test_models_of_one_kind_of_layer_through_the_scheduler(tmp_path, kernels, name):
+    """A model that keeps no pages at all, and one that keeps no state."""
+    folder = cases.write_folder(tmp_path / "m", ONE_KIND[name], seed=5)
+    config, tensors = plain.read_folder(folder)
+    prompts = [cases.tokens_of(n, 61, seed=60 + n) for n in (3, 11, 20)]
+    expected = []
+    for prompt in prompts:
+        tokens = list(prompt)
+        for _ in range(9):
+            tokens.append(int(torch.argmax(plain.forward(config, tensors, tokens)[0][-1])))
+        expected.append(tokens[len(prompt):])
+    runner = runner_for(folder, kernels, "float32", page=16, pages=16, slots=3)
+    core = EngineCore(runner, SchedulerConfig(max_batch_size=2, max_tokens_per_step=16), prefill_chunk_size=6)
+    assert core.generate(prompts, GenerationConfig(max_new_tokens=9)) == expected
+    assert len(runner.cache.sequences) == 0
     runner.close()
 
 
