@@ -27,6 +27,18 @@ def products_of_the_shipped_configurations():
     found = set()
     for path in sorted((ROOT / "configs").glob("*.json")):
         sizes = json.loads(path.read_text())
+        if "hidden_size" not in sizes:  # another architecture: every matrix of its own list of tensors, whole and cut over K
+            from llmserve_amd.registry import resolve_architecture
+
+            architecture = resolve_architecture(sizes)
+            spec = architecture.build_spec(architecture.config_class.from_dict(sizes))
+            for name, tensor in spec.tensors().items():
+                if len(tensor.shape) == 2 and name != spec.embedding_name:
+                    found.add((tensor.shape[0], tensor.shape[1], False, False))
+                    found.add((tensor.shape[0], tensor.shape[1], False, True))
+                    if name.endswith("mlp.gate"):
+                        found.add((2 * tensor.shape[0], tensor.shape[1], True, False))
+            continue
         hidden, heads, kv_heads = sizes["hidden_size"], sizes["num_attention_heads"], sizes["num_key_value_heads"]
         head_dim = sizes.get("head_dim") or hidden // heads
         found.add(((heads + 2 * kv_heads) * head_dim, hidden, False, False))
