@@ -168,6 +168,93 @@ __global__ __launch_bounds__(256) void expert_product_mfma_kernel(const bf16_t* 
   }
 }
 
+// The experts' products of a step of many rows (prompts): tiles of 128 rows of one expert by 128 columns, K in steps of 64
+// through LDS.  All 256 threads bring the two operand tiles from memory sixteen bytes at a time, eight threads a row (128
+// bytes in a row, where the kernel above asks for sixteen rows of 64 bytes an instruction and is bound by the address
+// path), two steps ahead in registers; the four waves (2 x 2) each make 64 x 64 of the result out of LDS.  Rows of LDS are
+// 144 bytes apart (banks).  Rows and columns beyond the tile's are read from the last valid one and never stored.
+#define TILED_ROWS 128
+#define TILED_K 64
+#define TILED_LINE 72  // elements: 64 and 8 of padding
+template <typename TO>
+__global__ __launch_bounds__(256) void expert_tiled_kernel(const bf16_t* __restrict__ x, const int* __restrict__ order, int top,
+                                                           const bf16_t* __restrict__ w, int outputs, int inner,
+                                                           const int* __restrict__ tiles, TO* __restrict__ out, int activation) {
+  __shared__ __attribute__((aligned(16))) bf16_t xs[TILED_ROWS * TILED_LINE], ws[TILED_ROWS * TILED_LINE];
+  const int* tile = tiles + 3 * (size_t)blockIdx.y;
+  const int expert = tile[0], first = tile[1], rows = tile[2];
+  if (rows == 0) return;
+  const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 15, g = lane >> 4;
+  const int wave_row = (wave >> 1) * 64, wave_col = (wave & 1) * 64;
+  const int col0 = blockIdx.x * TILED_ROWS;
+  const int piece = t % 8;  // which sixteen bytes of a row's 128 a step
+  const bf16_t* x_from[4];
+  const bf16_t* w_from[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = min(t / 8 + 32 * j, rows - 1), place = first + row;
+    x_from[j] = x + (size_t)(top > 0 ? order[place] / top : place) * inner + piece * 8;
+    const int n = min(col0 + t / 8 + 32 * j, outputs - 1);
+    w_from[j] = w + ((size_t)expert * outputs + n) * inner + piece * 8;
+  }
+  bf16x8 x_next[4], w_next[4], x_after[4], w_after[4];  // the next step's pieces, and the one's after it
+  const int second = min(TILED_K, inner - TILED_K);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    x_next[j] = *(const bf16x8*)x_from[j];
+    w_next[j] = *(const bf16x8*)w_from[j];
+    x_after[j] = *(const bf16x8*)(x_from[j] + second);
+    w_after[j] = *(const bf16x8*)(w_from[j] + second);
+  }
+  f32x4 acc[4][4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s)
+#pragma unroll
+    for (int u = 0; u < 4; ++u) acc[s][u] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < inner; k0 += TILED_K) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      *(bf16x8*)&xs[(t / 8 + 32 * j) * TILED_LINE + piece * 8] = x_next[j];
+      *(bf16x8*)&ws[(t / 8 + 32 * j) * TILED_LINE + piece * 8] = w_next[j];
+      x_next[j] = x_after[j];
+      w_next[j] = w_after[j];
+    }
+    __syncthreads();
+    const int ahead = min(k0 + 2 * TILED_K, inner - TILED_K);  // (in no branch; the last steps ask for the last again)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      x_after[j] = *(const bf16x8*)(x_from[j] + ahead);
+      w_after[j] = *(const bf16x8*)(w_from[j] + ahead);
+    }
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      bf16x8 a[4], b[4];
+#pragma unroll
+      for (int s = 0; s < 4; ++s) a[s] = *(const bf16x8*)&ws[(wave_col + s * 16 + r) * TILED_LINE + half * 32 + g * 8];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) b[u] = *(const bf16x8*)&xs[(wave_row + u * 16 + r) * TILED_LINE + half * 32 + g * 8];
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) acc[s][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s], b[u], acc[s][u], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int m = wave_row + u * 16 + r;
+    if (m >= rows) continue;
+    TO* dst = out + (size_t)(first + m) * outputs;
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = col0 + wave_col + s * 16 + g * 4 + i;
+        if (n < outputs) dst[n] = from_float<TO>(activation_of(activation, acc[s][u][i]));
+      }
+  }
+}
+
 // The experts' products of a step of few rows (decoding): every tile holds a few rows of one expert, and the product is a
 // stream of that expert's weights.  A workgroup owns 16 weight rows of one tile's expert and its four waves take the
 // 32-wide steps of K in turn (wave v the steps v, v + 4, ...), so that four times as many loads are under way as with a
@@ -369,7 +456,7 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_pairs_kernel(const int* __r
 extern "C" int llmserve_sort_pairs(const int* chosen, int pairs, int experts, int* place, int* order, int* tiles,
                                    int capacity, int tile_rows, hipStream_t stream) {
   if (pairs <= 0) return 0;
-  if (experts < 1 || experts > MAX_EXPERTS || (tile_rows != 16 && tile_rows != 64) ||
+  if (experts < 1 || experts > MAX_EXPERTS || (tile_rows != 16 && tile_rows != 64 && tile_rows != 128) ||
       capacity < (pairs + tile_rows - 1) / tile_rows + experts)
     return ERR_BAD_ARGUMENT;
   hipLaunchKernelGGL(sort_pairs_kernel, dim3(1), dim3(SORT_THREADS), 0, stream, chosen, pairs, experts, place, order, tiles, capacity,
@@ -409,14 +496,25 @@ __global__ __launch_bounds__(256) void expert_product_kernel(const TX* __restric
 }
 
 // x, w and the first product's result are of one type (bfloat16 or float32); the second product's result is float32.
-// `tile_rows` is what the tiles were made for: 16, or 64 (bfloat16 with a K in steps of 32 only: the matrix cores).
+// `tile_rows` is what the tiles were made for: 16; or, bfloat16 on the matrix cores only, 64 (K in steps of 32) or 128 (K in
+// steps of 64: operands through LDS).
 extern "C" int llmserve_expert_product(const void* x, int is_float, const int* order, int top, const void* w, int outputs,
                                        int inner, const int* tiles, int capacity, int tile_rows, void* out, int out_is_float,
                                        int activation, hipStream_t stream) {
   if (capacity <= 0) return 0;
   if (capacity > 65535 || outputs < 1 || inner < 1) return ERR_BAD_ARGUMENT;
+  if (!is_float && tile_rows == TILED_ROWS) {
+    if (inner % TILED_K) return ERR_BAD_ARGUMENT;
+    const dim3 through_lds((outputs + TILED_ROWS - 1) / TILED_ROWS, capacity);
+    if (out_is_float)
+      hipLaunchKernelGGL(expert_tiled_kernel<float>, through_lds, dim3(256), 0, stream, (const bf16_t*)x, order, top, (const bf16_t*)w,
+                         outputs, inner, tiles, (float*)out, activation);
+    else
+      hipLaunchKernelGGL(expert_tiled_kernel<bf16_t>, through_lds, dim3(256), 0, stream, (const bf16_t*)x, order, top, (const bf16_t*)w,
+                         outputs, inner, tiles, (bf16_t*)out, activation);
+    return LAUNCH_STATUS();
+  }
   if (!is_float && inner % 32 == 0) {
-    // a few tiles (decoding) stream their experts' weights: a tile of weight rows a wave, so that many workgroups share the stream
     if (tile_rows == 16 && capacity * ((outputs + 15) / 16) <= 8192) {
       // a few tiles (decoding) stream their experts' weights: sixteen weight rows a workgroup, K dealt out to its waves
       const dim3 streams((outputs + 15) / 16, capacity);

@@ -136,7 +136,7 @@ def test_join_activate_and_gated_add(kernels, dtype):
 @pytest.mark.parametrize("tokens,experts,top,hidden,size", [
     (1, 4, 4, 32, 16), (37, 8, 2, 96, 40), (200, 5, 3, 64, 72),
     # sizes in steps of 32: in bfloat16 the matrix cores, tiles of 16 rows for a few rows an expert and of 64 for many
-    (5, 8, 2, 64, 32), (300, 4, 2, 64, 96), (130, 3, 1, 320, 64),
+    (5, 8, 2, 64, 32), (300, 4, 2, 64, 96), (130, 3, 1, 320, 64), (700, 3, 2, 192, 320), (1000, 2, 1, 128, 64),
 ])
 def test_routed_experts(kernels, dtype, tokens, experts, top, hidden, size):
     torch.manual_seed(tokens)
