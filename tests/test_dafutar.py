@@ -315,3 +315,18 @@ def test_models_of_one_kind_of_layer_through_the_scheduler(tmp_path, name):
     core = EngineCore(runner, SchedulerConfig(max_batch_size=2, max_tokens_per_step=16), prefill_chunk_size=6)
     assert core.generate(prompts, GenerationConfig(max_new_tokens=5)) == expected
     assert len(runner.cache.sequences) == 0
+
+
+def test_the_command_line_writes_a_random_model_folder(tmp_path, capsys):
+    """`llmserve random-model` goes through the registry: a Dafutar config.json gives a folder that loads and runs."""
+    import json
+
+    from llmserve_amd.cli import main
+
+    (tmp_path / "config.json").write_text(json.dumps(cases.MIXED))
+    assert main(["random-model", "--config", str(tmp_path / "config.json"), "--output", str(tmp_path / "out"), "--seed", "5", "--std", "0.2"]) == 0
+    assert str(tmp_path / "out") in capsys.readouterr().out
+    tokens = cases.tokens_of(12, 61, seed=2)
+    want, _ = oracle(tmp_path / "out", tokens)
+    runner = runner_for(tmp_path / "out")
+    close(runner.step([StepEntry("a", tokens, range(12))], create_missing=True), want)
