@@ -55,13 +55,14 @@ class Kernels(Protocol):
 
     def paged_attention(
         self, qkv: torch.Tensor, layout: Any, batch: Any, cell: Any, scale: float, window: int | None, *,
-        score_slopes: torch.Tensor | None = None, soft_cap: float | None = None,
+        score_slopes: torch.Tensor | None = None, soft_cap: float | None = None, sinks: torch.Tensor | None = None,
     ) -> torch.Tensor:
         """Attention of the q heads of `qkv` over the cell's pages -> [T, heads * head_dim].
         Before the softmax a score s of a query at position p for a key at position k may be changed,
         for encodings and models that want it (Qwen2 wants neither): with `soft_cap`, to
         soft_cap * tanh(s / soft_cap); with `score_slopes` (float32, one per query head), by
-        - slope * (p - k) after that.  A library refuses what it cannot compute."""
+        - slope * (p - k) after that.  With `sinks` (float32, one per query head) the softmax's denominator
+        has exp(sink) more, once, with no value to it.  A library refuses what it cannot compute."""
 
     def rotate_store_attend(
         self, qkv: torch.Tensor, layout: Any, batch: Any, cell: Any,
@@ -144,7 +145,43 @@ class Kernels(Protocol):
         self, read: torch.Tensor, gates: torch.Tensor, gate_first: int, weight: torch.Tensor, eps: float, heads: int,
         vdim: int, activation: str,
     ) -> torch.Tensor:
-        """Per head: read / rms(read) * weight * act(gates[:, gate_first + h * vdim : + vdim]) -> run dtype [T, heads * vdim]."""
+        """Per head: read / rms(read) * weight * act(gates[:, gate_first + h * vdim : + vdim]) -> run dtype [T, heads * vdim];
+        act silu or sigmoid; weight of vdim for every head."""
+
+    # ------------------------------------------------------------------ norms on results, heads put together, linear attention
+
+    def stream_rows(self, hidden: torch.Tensor, delta: torch.Tensor | None) -> torch.Tensor:
+        """`hidden += delta` in place (float32), then the rows in the run dtype (in a float32 run the stream itself)."""
+
+    def add_normed(self, hidden: torch.Tensor, update: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+        """`hidden += u * rsqrt(mean(u^2) + eps) * weight` in place, u the float32 rows of `update` (its parts added
+        first); -> the new rows in the run dtype (in a float32 run the stream itself)."""
+
+    def assemble_heads(
+        self, x: torch.Tensor, q_first: int, k_first: int, v_first: int, heads: int, kv_heads: int, dim: int, vdim: int,
+        width: int, norm: str | None, q_weight: torch.Tensor | None, k_weight: torch.Tensor | None, eps: float,
+        table: torch.Tensor | None, rot_dims: int, other: torch.Tensor | None = None, other_first: int = 0, blend: float = 0.0,
+    ) -> torch.Tensor:
+        """From rows that hold `heads` queries and `kv_heads` keys of `dim` and `kv_heads` values of `vdim` (from the
+        columns q_first, k_first, v_first): rows [T, (heads + 2 kv_heads) * width] of queries, keys and values of
+        `width`, zeros beyond a head's own size.  Queries and keys are RMS-normed (`norm` "head": every head by
+        itself, weights of dim; "row": all query heads together and all key heads together, weights as long as
+        they; None), then their first `rot_dims` dimensions turned in adjacent pairs by the token's row of `table`
+        (float32 [T, rot_dims / 2, 2], cos and sin).  With `other`: v <- (1 - blend) v + blend * other[:, other_first : + kv_heads * vdim]."""
+
+    def scale_heads(self, x: torch.Tensor, heads: int, width: int, gates: torch.Tensor, gate_first: int, squash: str) -> torch.Tensor:
+        """x[:, h * width : (h + 1) * width] *= squash(gates[:, gate_first + h]) for every head, in place."""
+
+    def decay_attention(
+        self, x: torch.Tensor, q_first: int, k_first: int, v_first: int, heads: int, dim: int, vdim: int, decays: torch.Tensor,
+        activation: str, batch: Any, state: torch.Tensor,
+    ) -> torch.Tensor:
+        """q, k (heads of dim) and v (heads of vdim) are act of x's columns from q_first, k_first, v_first.  Per request
+        and head, token by token: S = decay_h S + k v^T; o = S^T q.  `state` float32 [slots, heads, dim, vdim] holds S
+        and is updated; decays float32 [heads].  -> float32 [T, heads * vdim]."""
+
+    def soft_cap(self, logits: torch.Tensor, cap: float) -> torch.Tensor:
+        """cap * tanh(logits / cap), in place (float32)."""
 
     # ------------------------------------------------------------------ routed experts
 

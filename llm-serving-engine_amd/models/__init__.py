@@ -1,3 +1,3 @@
-from . import dafutar, qwen2  # register Dafutar and Qwen2ForCausalLM
+from . import dafutar, qwen2, sozavik  # register Dafutar, Qwen2ForCausalLM and Sozavik
 
-__all__ = ["dafutar", "qwen2"]
+__all__ = ["dafutar", "qwen2", "sozavik"]

@@ -17,13 +17,15 @@ from .base import (
     TensorSpec,
 )
 from .norm import LayerNorm, LayerNormSpec, RMSNorm, RMSNormSpec
-from .position import HeadLayout, NoPositionSpec, PositionEncoding, Rotary, RotarySpec, YarnScaling, rotary_frequencies
+from .position import HeadLayout, NoPositionSpec, PositionEncoding, Rotary, RotarySpec, WavelengthScaling, YarnScaling, rotary_frequencies
 from .attention import Attention, AttentionSpec, Mixer
 from .feed_forward import FeedForward, GatedMLP, GatedMLPSpec
-from .block import Block, PreNormBlock, PreNormBlockSpec
-from .model import DecoderModel, JoinedPass, JoinedPassSpec, LayerDefinition, LayerRun, ModelSpec, NamedPart
+from .block import Block, OutputNormBlock, OutputNormBlockSpec, PreNormBlock, PreNormBlockSpec
+from .model import DecoderModel, JoinedPass, JoinedPassSpec, LayerDefinition, LayerRun, ModelSpec, NamedPart, SoftCap, SoftCapSpec
 from .latent_attention import LatentAttention, LatentAttentionSpec
 from .delta import GatedDelta, GatedDeltaSpec
 from .experts import RoutedExperts, RoutedExpertsSpec
+from .normed_attention import NormedAttention, NormedAttentionSpec
+from .decay_attention import DecayAttention, DecayAttentionSpec
 
 __all__ = [name for name in dir() if not name.startswith("_")]

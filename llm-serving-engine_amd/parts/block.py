@@ -77,3 +77,38 @@ class PreNormBlock(Block):
             return mixed
         normed = self.feed_forward_norm.forward(hidden, mixed)
         return self.feed_forward.forward(normed, batch)
+
+
+@dataclass(frozen=True)
+class OutputNormBlockSpec:
+    """h += norm(mixer(h)); h += norm(feed_forward(h)): the sublayers read the stream itself, and the norms act on
+    what they return.  Fields as in `PreNormBlockSpec`."""
+
+    mixer_norm: Any
+    mixer: Any
+    feed_forward_norm: Any
+    feed_forward: Any
+    mixer_norm_name: str = "norm1."
+    mixer_name: str = "mix."
+    feed_forward_norm_name: str = "norm2."
+    feed_forward_name: str = "mlp."
+    kind: str = "outnorm"
+
+
+@BLOCKS.register("outnorm")
+class OutputNormBlock(PreNormBlock):
+    """The stream is float32; a sublayer reads it rounded to the run dtype, and the kernel that adds a normed result to
+    the stream also writes that rounded copy for the next sublayer (of this layer or of the next one, which finds it
+    on the step).  Nothing is left pending: the block returns None."""
+
+    def forward(self, hidden, delta, batch, cell):
+        kept = batch.computed.get("stream rows")
+        if delta is None and kept is not None and kept[0] is hidden:
+            rows = kept[1]
+        else:
+            rows = self.kernels.stream_rows(hidden, delta)
+        rows = self.mixer_norm.add_normed(hidden, self.mixer.forward(rows, batch, cell))
+        if self.feed_forward is not None:
+            rows = self.feed_forward_norm.add_normed(hidden, self.feed_forward.forward(rows, batch))
+        batch.computed["stream rows"] = (hidden, rows)
+        return None

@@ -195,3 +195,33 @@ class JoinedPass:
     def forward(self, hidden, delta, embedded, batch, number: int):
         both = self.kernels.join_rows(hidden, delta, embedded)  # [T, 2 hidden] in the run dtype
         return self.kernels.linear(both, self.products[number], out_dtype=torch.float32)
+
+
+@dataclass(frozen=True)
+class SoftCapSpec:
+    cap: float
+    kind: str = "soft_cap"
+
+
+@LOGIT_PARTS.register("soft_cap")
+class SoftCap:
+    """logits <- cap * tanh(logits / cap), in place on the wanted rows."""
+
+    replayable = True
+
+    @classmethod
+    def tensors(cls, spec: SoftCapSpec) -> dict[str, TensorSpec]:
+        return {}
+
+    @classmethod
+    def cache_need(cls, spec: SoftCapSpec) -> None:
+        return None
+
+    def __init__(self, spec: SoftCapSpec, tensors, kernels) -> None:
+        if not spec.cap > 0:
+            raise ValueError("soft cap: the cap is positive")
+        self.spec = spec
+        self.kernels = kernels
+
+    def forward(self, logits, batch):
+        return self.kernels.soft_cap(logits, self.spec.cap)

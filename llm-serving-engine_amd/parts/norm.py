@@ -11,8 +11,11 @@ from .base import NORMS, Part, TensorSpec
 
 @dataclass(frozen=True)
 class RMSNormSpec:
+    """`weight_name` is the tensor's name below the part's prefix (a model whose files call it otherwise says so)."""
+
     size: int
     eps: float
+    weight_name: str = "weight"
     kind: str = "rmsnorm"
 
 
@@ -24,15 +27,21 @@ class RMSNorm(Part):
 
     @classmethod
     def tensors(cls, spec: RMSNormSpec) -> dict[str, TensorSpec]:
-        return {"weight": TensorSpec((spec.size,), role="norm")}
+        return {spec.weight_name: TensorSpec((spec.size,), role="norm")}
 
     def __init__(self, spec: RMSNormSpec, tensors, kernels) -> None:
         super().__init__(spec, tensors, kernels)
-        self.weight = tensors["weight"]
+        self.weight = tensors[spec.weight_name]
 
     def forward(self, hidden: torch.Tensor, delta: torch.Tensor | None) -> torch.Tensor:
         """Adds `delta` into `hidden` (in place) and returns the normed rows in the run dtype."""
         return self.kernels.add_rms_norm(hidden, delta, self.weight, self.spec.eps)
+
+    def add_normed(self, hidden: torch.Tensor, update: torch.Tensor) -> torch.Tensor:
+        """The norm on a sublayer's output instead of its input: `hidden += update * rsqrt(mean(update^2) + eps) *
+        weight` in place (float32; `update` may be partial sums, which are added first), and returns the new stream in
+        the run dtype, as the next sublayer reads it."""
+        return self.kernels.add_normed(hidden, update, self.weight, self.spec.eps)
 
 
 @dataclass(frozen=True)

@@ -107,13 +107,32 @@ class YarnScaling:
     slow: float
 
 
-def rotary_frequencies(dims: int, theta: float, scaling: YarnScaling | None = None) -> tuple[torch.Tensor, float]:
+@dataclass(frozen=True)
+class WavelengthScaling:
+    """Frequencies stretched by wavelength: a pair whose wavelength is below `original / high` keeps its frequency,
+    one above `original / low` has it divided by `factor`, and between the two the divided and the plain frequency
+    are blended, s = (original / wavelength - low) / (high - low) of the plain one.  Cosines and sines stay as they are."""
+
+    factor: float
+    low: float
+    high: float
+    original: float
+
+
+def rotary_frequencies(dims: int, theta: float, scaling: "YarnScaling | WavelengthScaling | None" = None) -> tuple[torch.Tensor, float]:
     """(float32 frequencies [dims / 2] of pair i, theta^(-2i / dims), stretched by `scaling`; what the cosines
     and sines are multiplied by).  Computed in float64 and rounded once."""
     index = torch.arange(dims // 2, dtype=torch.float64)
     plain = float(theta) ** (-2.0 * index / dims)
     if scaling is None:
         return plain.to(torch.float32), 1.0
+    if isinstance(scaling, WavelengthScaling):
+        wavelength = 2.0 * math.pi / plain
+        share = ((scaling.original / wavelength - scaling.low) / (scaling.high - scaling.low)).clamp(0.0, 1.0)
+        blended = (1.0 - share) * plain / scaling.factor + share * plain
+        stretched = torch.where(wavelength < scaling.original / scaling.high, plain,
+                                torch.where(wavelength > scaling.original / scaling.low, plain / scaling.factor, blended))
+        return stretched.to(torch.float32), 1.0
 
     def turning_pair(turns: float) -> float:  # the (fractional) dimension whose wavelength makes `turns` turns over the original context
         return dims * math.log(scaling.original / (2.0 * math.pi * turns)) / (2.0 * math.log(theta))

@@ -88,7 +88,7 @@ class TorchKernels:
             cell.put_key_rows(pages, offsets, view[:, heads : heads + kv_heads])  # pages are [kv, dim / w, offset, w]
             cell.put_value_rows(pages, offsets, view[:, heads + kv_heads :])  # pages are [kv, offset / v, dim, v]
 
-    def paged_attention(self, qkv, layout, batch, cell, scale, window, *, score_slopes=None, soft_cap=None):
+    def paged_attention(self, qkv, layout, batch, cell, scale, window, *, score_slopes=None, soft_cap=None, sinks=None):
         tokens = qkv.shape[0]
         heads, kv_heads, dim = layout.num_heads, layout.num_kv_heads, layout.head_dim
         queries = qkv.view(tokens, heads + 2 * kv_heads, dim)[:, :heads].float()
@@ -111,7 +111,11 @@ class TorchKernels:
                     scores = soft_cap * torch.tanh(scores / soft_cap)
                 if score_slopes is not None:
                     scores = scores - score_slopes.float().view(-1, 1) * (position - where).float()
-                out[row] = torch.einsum("hn,nhd->hd", torch.softmax(scores, dim=-1), values)
+                if sinks is not None:  # a column more in the softmax, with no value
+                    scores = torch.cat([scores, sinks.float().view(-1, 1)], dim=1)
+                    out[row] = torch.einsum("hn,nhd->hd", torch.softmax(scores, dim=-1)[:, :-1], values)
+                else:
+                    out[row] = torch.einsum("hn,nhd->hd", torch.softmax(scores, dim=-1), values)
                 row += 1
         return out.reshape(tokens, heads * dim).to(self.dtype)
 
@@ -256,12 +260,80 @@ class TorchKernels:
         return out.reshape(tokens, heads * vdim)
 
     def gated_head_norm(self, read, gates, gate_first, weight, eps, heads, vdim, activation):
-        assert activation == "silu"
+        squash = {"silu": torch.nn.functional.silu, "sigmoid": torch.sigmoid}[activation]
         tokens = read.shape[0]
         rows = read.view(tokens, heads, vdim)
         normed = rows * torch.rsqrt(rows.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
-        gate = torch.nn.functional.silu(gates[:, gate_first : gate_first + heads * vdim].float()).view(tokens, heads, vdim)
+        gate = squash(gates[:, gate_first : gate_first + heads * vdim].float()).view(tokens, heads, vdim)
         return (normed * gate).reshape(tokens, heads * vdim).to(self.dtype)
+
+    # ------------------------------------------------------------------ norms on results, heads put together, linear attention
+
+    def stream_rows(self, hidden, delta):
+        if delta is not None:
+            hidden += delta if delta.ndim == 2 else delta.sum(0)
+        return hidden if self.dtype == torch.float32 else hidden.to(self.dtype)
+
+    def add_normed(self, hidden, update, weight, eps):
+        u = update if update.ndim == 2 else update.sum(0)
+        hidden += u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+        return hidden if self.dtype == torch.float32 else hidden.to(self.dtype)
+
+    def assemble_heads(self, x, q_first, k_first, v_first, heads, kv_heads, dim, vdim, width, norm, q_weight, k_weight, eps,
+                       table, rot_dims, other=None, other_first=0, blend=0.0):
+        tokens = x.shape[0]
+        out = torch.zeros((tokens, heads + 2 * kv_heads, width))
+
+        def normed_turned(first, count, weight):
+            part = x[:, first : first + count * dim].float()
+            if norm == "row":
+                part = part * torch.rsqrt(part.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+            part = part.reshape(tokens, count, dim)
+            if norm == "head":
+                part = part * torch.rsqrt(part.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+            if rot_dims:
+                cos, sin = table[:, None, :, 0], table[:, None, :, 1]
+                a, b = part[..., 0:rot_dims:2], part[..., 1:rot_dims:2]
+                turned = part.clone()
+                turned[..., 0:rot_dims:2] = a * cos - b * sin
+                turned[..., 1:rot_dims:2] = b * cos + a * sin
+                part = turned
+            return part
+
+        out[:, :heads, :dim] = normed_turned(q_first, heads, q_weight)
+        out[:, heads : heads + kv_heads, :dim] = normed_turned(k_first, kv_heads, k_weight)
+        values = x[:, v_first : v_first + kv_heads * vdim].float()
+        if other is not None:
+            values = (1.0 - blend) * values + blend * other[:, other_first : other_first + kv_heads * vdim].float()
+        out[:, heads + kv_heads :, :vdim] = values.reshape(tokens, kv_heads, vdim)
+        return out.reshape(tokens, -1).to(self.dtype)
+
+    def scale_heads(self, x, heads, width, gates, gate_first, squash):
+        assert squash == "sigmoid"
+        gate = torch.sigmoid(gates[:, gate_first : gate_first + heads].float())
+        x.copy_((x.float().view(x.shape[0], heads, width) * gate[:, :, None]).reshape(x.shape).to(x.dtype))
+        return x
+
+    def decay_attention(self, x, q_first, k_first, v_first, heads, dim, vdim, decays, activation, batch, state):
+        assert activation == "silu"
+        tokens = x.shape[0]
+        act = torch.nn.functional.silu
+        q = act(x[:, q_first : q_first + heads * dim].float()).view(tokens, heads, dim)
+        k = act(x[:, k_first : k_first + heads * dim].float()).view(tokens, heads, dim)
+        v = act(x[:, v_first : v_first + heads * vdim].float()).view(tokens, heads, vdim)
+        out = torch.zeros((tokens, heads, vdim))
+        row = 0
+        for chunk in batch.chunks:
+            S = state[chunk.slot]  # [heads, dim, vdim], updated in place
+            for t in range(row, row + chunk.count):
+                S *= decays.float().view(heads, 1, 1)
+                S += torch.einsum("hd,hv->hdv", k[t], v[t])
+                out[t] = torch.einsum("hdv,hd->hv", S, q[t])
+            row += chunk.count
+        return out.reshape(tokens, heads * vdim)
+
+    def soft_cap(self, logits, cap):
+        return logits.copy_(cap * torch.tanh(logits / cap))
 
     # ------------------------------------------------------------------ routed experts
 
