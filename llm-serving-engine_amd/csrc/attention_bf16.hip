@@ -98,6 +98,7 @@ struct FusedDecode {          // what the kernel needs to rotate and store; unus
 struct ScoreChange {          // unused unless CHANGED
   const float* slopes;        // [heads], or null
   float soft_cap;             // 0: none
+  const float* sinks;         // [heads], or null: exp(sink) more in a head's denominator, once, with no value to it
 };
 
 // One step's operands as a lane holds them: its slices of the K rows of the two 16-row tiles and,
@@ -591,7 +592,15 @@ __global__ __launch_bounds__(WAVES * 64, (COLUMN_TILES > 2 || HEAD_DIM > 192 || 
       const int head = kv_head * group + head_tile * 16 + head_here;
       const size_t row = (size_t)row0 + token;
       if (splits == 1) {
-        const float inverse = total > 0.f ? 1.f / total : 0.f;
+        float shrink = 1.f;
+        if constexpr (CHANGED) {
+          if (change.sinks) {  // (in units of log2, as the maxima are)
+            const float sink = change.sinks[head] * 1.44269504088896f, top = fmaxf(best, sink);
+            shrink = __builtin_amdgcn_exp2f(best - top);
+            total = total * shrink + __builtin_amdgcn_exp2f(sink - top);
+          }
+        }
+        const float inverse = total > 0.f ? shrink / total : 0.f;
         const bf16x4 rounded = {(bf16_t)(merged[0] * inverse), (bf16_t)(merged[1] * inverse), (bf16_t)(merged[2] * inverse),
                                 (bf16_t)(merged[3] * inverse)};
         *(bf16x4*)(out + (row * heads + head) * D + d4) = rounded;
@@ -650,13 +659,20 @@ __device__ __forceinline__ float merge_some(const float* acc, int first, int spl
 // out[d] = sum_s acc_s[d] w_s / sum_s l_s w_s of the splits whose maxima and sums lie at `ml` and partial sums at
 // `acc`, for the dimensions threadIdx.x, threadIdx.x + blockDim.x, ...; every lane of every wave must call it (the
 // weights pass between lanes)
-__device__ __forceinline__ void merge_splits(const float* ml, const float* acc, int splits, bf16_t* out) {
+// (`sink`: the head's sink in units of log2, or -INFINITY for none)
+__device__ __forceinline__ void merge_splits(const float* ml, const float* acc, int splits, bf16_t* out, float sink = -INFINITY) {
   const int lane = threadIdx.x & (WAVE - 1);
   const float2 mine = lane < splits ? *(const float2*)(ml + (size_t)lane * 2) : make_float2(-INFINITY, 0.f);
   const float best = wave_max(mine.x);
   const float weight = mine.x == -INFINITY ? 0.f : exp2f(mine.x - best);  // a split that saw no key counts nothing
-  const float total = wave_sum(mine.y * weight);                          // (lanes beyond the splits add 0)
-  const float inverse = total > 0.f ? 1.f / total : 0.f;
+  float total = wave_sum(mine.y * weight);                                // (lanes beyond the splits add 0)
+  float shrink = 1.f;
+  if (sink > -INFINITY) {
+    const float top = fmaxf(best, sink);
+    shrink = exp2f(best - top);
+    total = total * shrink + exp2f(sink - top);
+  }
+  const float inverse = total > 0.f ? shrink / total : 0.f;
   for (int d0 = 0; d0 < D; d0 += blockDim.x) {  // (the same trips for all lanes: those beyond D read D - 1 and store nothing)
     const int d = d0 + threadIdx.x;
     const float* mine_acc = acc + min(d, D - 1);
@@ -672,9 +688,11 @@ __device__ __forceinline__ void merge_splits(const float* ml, const float* acc, 
 // they are many: a prompt portion's 24,576 pairs in four splits 12 us against 15)
 __global__ __launch_bounds__(MERGE_THREADS) void attention_merge_kernel(const float* __restrict__ partial_acc,
                                                                         const float* __restrict__ partial_ml,
-                                                                        bf16_t* __restrict__ out, int splits) {
+                                                                        bf16_t* __restrict__ out, int splits,
+                                                                        const float* __restrict__ sinks, int heads) {
   const size_t pair = blockIdx.x;  // row * heads + head
-  merge_splits(partial_ml + pair * splits * 2, partial_acc + pair * splits * D, splits, out + pair * D);
+  const float sink = sinks ? sinks[pair % heads] * 1.44269504088896f : -INFINITY;
+  merge_splits(partial_ml + pair * splits * 2, partial_acc + pair * splits * D, splits, out + pair * D, sink);
 }
 
 // The same for partial results that are kept by work item: workgroup (item, head) merges the item's tokens one
@@ -683,20 +701,23 @@ __global__ __launch_bounds__(MERGE_THREADS) void attention_merge_items_kernel(co
                                                                               const float* __restrict__ partial_ml,
                                                                               bf16_t* __restrict__ out,
                                                                               const int* __restrict__ work, int splits,
-                                                                              int heads, int group, int tokens_per_tile) {
+                                                                              int heads, int group, int tokens_per_tile,
+                                                                              const float* __restrict__ sinks) {
   const int* item = work + (size_t)blockIdx.x * 4;
   const int tokens = group <= 16 ? (item[2] + item[3] + group - 1) / group : item[3];
   const int head = blockIdx.y;
+  const float sink = sinks ? sinks[head] * 1.44269504088896f : -INFINITY;
   for (int token = 0; token < tokens; ++token) {
     const size_t kept_as = ((size_t)blockIdx.x * tokens_per_tile + token) * heads + head;
     const size_t pair = ((size_t)item[1] + token) * heads + head;
-    merge_splits(partial_ml + kept_as * splits * 2, partial_acc + kept_as * splits * D, splits, out + pair * D);
+    merge_splits(partial_ml + kept_as * splits * 2, partial_acc + kept_as * splits * D, splits, out + pair * D, sink);
   }
 }
 
-static int launch_merge(float* partial_acc, float* partial_ml, void* out, int splits, size_t pairs, hipStream_t stream) {
+static int launch_merge(float* partial_acc, float* partial_ml, void* out, int splits, size_t pairs, hipStream_t stream,
+                        const float* sinks = nullptr, int heads = 1) {
   hipLaunchKernelGGL(attention_merge_kernel, dim3((unsigned)pairs), dim3(pairs >= 4096 ? WAVE : MERGE_THREADS), 0, stream,
-                     partial_acc, partial_ml, (bf16_t*)out, splits);
+                     partial_acc, partial_ml, (bf16_t*)out, splits, sinks, heads);
   return LAUNCH_STATUS();
 }
 
@@ -979,7 +1000,7 @@ static int launch_tiles(const void* qkv, int row_width, void* out, float* partia
                         void* keys, void* values, const int* block_tables, int table_width,
                         const int* positions, const int* work, int tiles, int heads, int kv_heads,
                         int tokens_per_tile, int page_size, float scale, int window, int splits, FusedDecode fused,
-                        hipStream_t stream, ScoreChange change = {nullptr, 0.f}) {
+                        hipStream_t stream, ScoreChange change = {nullptr, 0.f, nullptr}) {
   const int group = heads / kv_heads;
   const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
   const int head_tiles = (group + 15) / 16;
@@ -1026,18 +1047,18 @@ extern "C" int llmserve_attention_can_fuse(int pairing) {
 // weights, and partial_ml [heads][splits][16 rows][2] holds each split's maximum (in units of log2) and sum of
 // weights.
 // `slopes` (float32 [heads], or null) and `soft_cap` (0 for none) change the scores before the softmax (see the head of
-// this file); not together with `fuse` & 1.
+// this file), `sinks` (float32 [heads], or null) add exp(sink) to a head's denominator; not together with `fuse` & 1.
 extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* out, float* partial_acc,
                                         float* partial_ml, void* keys, void* values,
                                         const int* block_tables, int table_width, const int* positions,
                                         const int* work, int tiles, int column_tiles, int rows, int heads,
                                         int kv_heads, int page_size, float scale, int window, int splits, int fuse,
                                         const float* table, int pairing, const int* slots, const float* slopes,
-                                        float soft_cap, hipStream_t stream) {
+                                        float soft_cap, const float* sinks, hipStream_t stream) {
   if (tiles <= 0) return 0;
-  const bool changed = slopes != nullptr || soft_cap > 0.f;
-  if (soft_cap < 0.f || (changed && (fuse & 1))) return ERR_BAD_ARGUMENT;
-  const ScoreChange change = {slopes, soft_cap};
+  const bool changed = slopes != nullptr || soft_cap > 0.f || sinks != nullptr;
+  if (soft_cap < 0.f || (changed && (fuse & 1)) || (sinks && (fuse & 2))) return ERR_BAD_ARGUMENT;
+  const ScoreChange change = {slopes, soft_cap, sinks};
   if (heads % kv_heads || page_size % 8 || splits < 1 || splits > MERGE_SPLITS_MAX || (splits > 1 && (!partial_acc || !partial_ml)))
     return ERR_BAD_ARGUMENT;
   if ((long)kv_heads * page_size * D >= (1L << 31)) return ERR_BAD_ARGUMENT;  // a page's elements are counted in 32 bits
@@ -1078,8 +1099,8 @@ extern "C" int llmserve_attention_tiles(const void* qkv, int row_width, void* ou
   if (status != 0 || splits == 1 || unmerged) return status;
   if (by_item) {
     hipLaunchKernelGGL(attention_merge_items_kernel, dim3(tiles, heads), dim3(MERGE_THREADS), 0, stream, partial_acc, partial_ml,
-                       (bf16_t*)out, work, splits, heads, group, tokens_per_tile);
+                       (bf16_t*)out, work, splits, heads, group, tokens_per_tile, sinks);
     return LAUNCH_STATUS();
   }
-  return launch_merge(partial_acc, partial_ml, out, splits, (size_t)rows * heads, stream);
+  return launch_merge(partial_acc, partial_ml, out, splits, (size_t)rows * heads, stream, sinks, heads);
 }

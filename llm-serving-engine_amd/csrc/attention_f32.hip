@@ -5,7 +5,9 @@
 // remains for head sizes that are no multiple of 16 and pages that are no multiple of 4.
 // Two things may change a score before the softmax, for position encodings and models that want them
 // (the reference has neither): `soft_cap` > 0 squashes it to cap * tanh(score / cap), and `slopes` (one
-// per query head) then adds -slope * (query position - key position).
+// per query head) then adds -slope * (query position - key position).  With `sinks` (one per query head) the
+// softmax's denominator has exp(sink) more, once, with no value to it; it is added where a column's sums are final
+// (in the kernel that merges key splits, where there are splits).
 //
 // The unit of work is an item: up to 16 * COLUMN_TILES "columns", the (token, query head) pairs of
 // consecutive tokens of one request that share one kv head, running through the tokens head by head so
@@ -46,7 +48,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_f32_kernel(
     float* __restrict__ partial_ml, const float* __restrict__ keys, const float* __restrict__ values,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ positions,
     const int* __restrict__ work, int heads, int kv_heads, int page_size, float scale_log2, int window, int splits,
-    int columns_total, const float* __restrict__ slopes, float soft_cap) {
+    int columns_total, const float* __restrict__ slopes, float soft_cap, const float* __restrict__ sinks) {
   __shared__ float wave_max[WAVES][COLUMN_TILES][16];
   __shared__ float wave_sum[WAVES][COLUMN_TILES][16];
   __shared__ __attribute__((aligned(16))) float merged[COLUMN_TILES][D_STEPS][64][4];
@@ -240,7 +242,13 @@ __global__ __launch_bounds__(WAVES * 64) void attention_f32_kernel(
     for (int s = wave; s < D_STEPS; s += WAVES) {
       f32x4 result = *(const f32x4*)merged[t][s][lane];
       if (splits == 1) {
-        const float scale = total_sum[t] > 0.f ? 1.f / total_sum[t] : 0.f;
+        float sum = total_sum[t], shrink = 1.f;
+        if (CHANGED && sinks) {  // (in units of log2, as the maxima are)
+          const float sink = sinks[head[t]] * 1.4426950408889634f, top = fmaxf(total_max[t], sink);
+          shrink = exp2f(total_max[t] - top);
+          sum = sum * shrink + exp2f(sink - top);
+        }
+        const float scale = sum > 0.f ? shrink / sum : 0.f;
 #pragma unroll
         for (int e = 0; e < 4; ++e) result[e] *= scale;
         *(f32x4*)(out + column * D + 16 * s + 4 * g) = result;
@@ -281,15 +289,22 @@ __device__ __forceinline__ float merge_some(const float* acc, size_t split_strid
 __global__ __launch_bounds__(MERGE_THREADS) void attention_f32_merge_kernel(float* __restrict__ out,
                                                                            const float* __restrict__ partial_acc,
                                                                            const float* __restrict__ partial_ml,
-                                                                           int splits, int columns_total) {
+                                                                           int splits, int columns_total,
+                                                                           const float* __restrict__ sinks, int heads) {
   const size_t column = blockIdx.x;
   const int lane = threadIdx.x & 63, d = threadIdx.x;
   const float2 mine = lane < splits ? *(const float2*)(partial_ml + ((size_t)lane * columns_total + column) * 2)
                                     : make_float2(-INFINITY, 0.f);
   const float best = wave_max(mine.x);
   const float weight = mine.x == -INFINITY ? 0.f : exp2f(mine.x - best);  // a split that saw no key counts nothing
-  const float total = wave_sum(mine.y * weight);                          // (lanes beyond the splits add 0)
-  const float inverse = total > 0.f ? 1.f / total : 0.f;
+  float total = wave_sum(mine.y * weight);                                // (lanes beyond the splits add 0)
+  float shrink = 1.f;
+  if (sinks) {
+    const float sink = sinks[column % heads] * 1.4426950408889634f, top = fmaxf(best, sink);
+    shrink = exp2f(best - top);
+    total = total * shrink + exp2f(sink - top);
+  }
+  const float inverse = total > 0.f ? shrink / total : 0.f;
   const float* acc = partial_acc + column * D + min(d, D - 1);
   const size_t split_stride = (size_t)columns_total * D;
   float sum = 0.f;
@@ -302,13 +317,13 @@ __global__ __launch_bounds__(MERGE_THREADS) void attention_f32_merge_kernel(floa
 // qkv [tokens, row_width] float32 with the queries in front (heads * D), out [tokens, heads * D]; key pages in
 // pieces ([page, kv_head, D / 8, offset, 8]), value pages transposed in pieces of eight keys ([page, kv_head,
 // page_size / 8, D, 8]; common.h: value_element); work [items, 4].
-// column_tiles 1 or 2; page_size a multiple of 4; slopes float32 [heads] or null, soft_cap 0 for none.  With splits > 1: partial_acc float32 [splits, tokens * heads, D]
+// column_tiles 1 or 2; page_size a multiple of 4; slopes and sinks float32 [heads] or null, soft_cap 0 for none.  With splits > 1: partial_acc float32 [splits, tokens * heads, D]
 // and partial_ml [splits, tokens * heads, 2]; every column of the step must belong to an item.
 extern "C" int llmserve_attention_f32(const float* qkv, int row_width, float* out, float* partial_acc, float* partial_ml,
                                       const float* keys, const float* values, const int* block_tables, int table_width,
                                       const int* positions, const int* work, int items, int column_tiles, int tokens,
                                       int heads, int kv_heads, int page_size, float scale, int window, int splits,
-                                      const float* slopes, float soft_cap, hipStream_t stream) {
+                                      const float* slopes, float soft_cap, const float* sinks, hipStream_t stream) {
   if (items <= 0 || tokens <= 0) return 0;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || page_size <= 0 || page_size % 4 || splits < 1 ||
       splits > MERGE_SPLITS_MAX || (column_tiles != 1 && column_tiles != 2) || (splits > 1 && (!partial_acc || !partial_ml)))
@@ -316,11 +331,11 @@ extern "C" int llmserve_attention_f32(const float* qkv, int row_width, float* ou
   const float scale_log2 = scale * 1.4426950408889634f;
   const int columns_total = tokens * heads;
   dim3 grid(items, kv_heads, splits);
-  const bool changed = slopes != nullptr || soft_cap > 0.f;
+  const bool changed = slopes != nullptr || soft_cap > 0.f || sinks != nullptr;
 #define LAUNCH_ATTENTION_F32(TILES, CHANGED)                                                                          \
   hipLaunchKernelGGL((attention_f32_kernel<TILES, CHANGED>), grid, dim3(WAVES * 64), 0, stream, qkv, row_width, out,   \
                      partial_acc, partial_ml, keys, values, block_tables, table_width, positions, work, heads,        \
-                     kv_heads, page_size, scale_log2, window, splits, columns_total, slopes, soft_cap)
+                     kv_heads, page_size, scale_log2, window, splits, columns_total, slopes, soft_cap, sinks)
   if (column_tiles == 1 && !changed) LAUNCH_ATTENTION_F32(1, false);
   else if (column_tiles == 1) LAUNCH_ATTENTION_F32(1, true);
   else if (!changed) LAUNCH_ATTENTION_F32(2, false);
@@ -329,6 +344,6 @@ extern "C" int llmserve_attention_f32(const float* qkv, int row_width, float* ou
   int status = LAUNCH_STATUS();
   if (status != 0 || splits == 1) return status;
   hipLaunchKernelGGL(attention_f32_merge_kernel, dim3(columns_total), dim3(MERGE_THREADS), 0, stream, out, partial_acc, partial_ml,
-                     splits, columns_total);
+                     splits, columns_total, sinks, heads);
   return LAUNCH_STATUS();
 }

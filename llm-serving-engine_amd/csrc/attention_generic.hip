@@ -8,7 +8,8 @@
 // Two things may change a score before the softmax, for position encodings and models that want
 // them (the reference has neither): `soft_cap` > 0 squashes it to cap * tanh(score / cap), and
 // `slopes` (one per query head) then adds -slope * (query position - key position), a bias that
-// grows with distance.
+// grows with distance.  With `sinks` (one per query head) the softmax's denominator has exp(sink) more, once, with
+// no value to it: a key that is not there.
 #include "common.h"
 
 #define KEYS_PER_TILE 128
@@ -19,7 +20,7 @@ __global__ __launch_bounds__(KEYS_PER_TILE) void attention_generic_kernel(
     const T* __restrict__ qkv, int row_width, T* __restrict__ out, const T* __restrict__ keys,
     const T* __restrict__ values, const int* __restrict__ block_tables, int table_width,
     const int* __restrict__ token_sequence, const int* __restrict__ positions, int heads, int kv_heads, int dim,
-    int page_size, float scale, int window, const float* __restrict__ slopes, float soft_cap) {
+    int page_size, float scale, int window, const float* __restrict__ slopes, float soft_cap, const float* __restrict__ sinks) {
   __shared__ float query[MAX_DIM];
   __shared__ float weights[KEYS_PER_TILE];
   __shared__ float shared[17];
@@ -77,10 +78,16 @@ __global__ __launch_bounds__(KEYS_PER_TILE) void attention_generic_kernel(
     }
     __syncthreads();
   }
+  float shrink = 1.f;  // what the results are multiplied by where the sink's exponential is the largest
+  if (sinks) {
+    const float sink = sinks[head], top = fmaxf(running_max, sink);
+    shrink = expf(running_max - top);
+    running_sum = running_sum * shrink + expf(sink - top);
+  }
   T* o = out + ((size_t)token * heads + head) * dim;
   for (int i = 0; i < per_thread; ++i) {
     const int d = threadIdx.x + i * KEYS_PER_TILE;
-    if (d < dim) o[d] = from_float<T>(acc[i] / running_sum);
+    if (d < dim) o[d] = from_float<T>(acc[i] * shrink / running_sum);
   }
 }
 
@@ -88,17 +95,17 @@ extern "C" int llmserve_attention_generic(const void* qkv, int row_width, void* 
                                           const void* values, const int* block_tables, int table_width,
                                           const int* token_sequence, const int* positions, int tokens, int heads,
                                           int kv_heads, int dim, int page_size, float scale, int window,
-                                          const float* slopes, float soft_cap, hipStream_t stream) {
+                                          const float* slopes, float soft_cap, const float* sinks, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (dim > MAX_DIM || dim <= 0 || heads % kv_heads || page_size <= 0) return ERR_BAD_ARGUMENT;
   dim3 grid(tokens, heads);
   if (is_float)
     hipLaunchKernelGGL(attention_generic_kernel<float>, grid, dim3(KEYS_PER_TILE), 0, stream, (const float*)qkv,
                        row_width, (float*)out, (const float*)keys, (const float*)values, block_tables, table_width,
-                       token_sequence, positions, heads, kv_heads, dim, page_size, scale, window, slopes, soft_cap);
+                       token_sequence, positions, heads, kv_heads, dim, page_size, scale, window, slopes, soft_cap, sinks);
   else
     hipLaunchKernelGGL(attention_generic_kernel<bf16_t>, grid, dim3(KEYS_PER_TILE), 0, stream, (const bf16_t*)qkv,
                        row_width, (bf16_t*)out, (const bf16_t*)keys, (const bf16_t*)values, block_tables, table_width,
-                       token_sequence, positions, heads, kv_heads, dim, page_size, scale, window, slopes, soft_cap);
+                       token_sequence, positions, heads, kv_heads, dim, page_size, scale, window, slopes, soft_cap, sinks);
   return LAUNCH_STATUS();
 }

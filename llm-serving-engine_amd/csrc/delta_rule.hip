@@ -472,31 +472,35 @@ extern "C" int llmserve_conv_gated_delta_rule(const void* x, int is_float, int x
 // out[t, h, :] = read[t, h, :] * rsqrt(mean(read[t, h, :]^2) + eps) * weight * silu(gates[t, gate_first + h * vdim + :]),
 // one wave per (token, head).
 template <typename T>
-__global__ __launch_bounds__(64) void gated_head_norm_kernel(const float* __restrict__ read, const T* __restrict__ gates,
+__global__ __launch_bounds__(512) void gated_head_norm_kernel(const float* __restrict__ read, const T* __restrict__ gates,
                                                              int gate_stride, int gate_first, const void* __restrict__ weight,
-                                                             int weight_is_float, float eps, int vdim, T* __restrict__ out) {
+                                                             int weight_is_float, float eps, int vdim, int squash,
+                                                             T* __restrict__ out) {
   const size_t base = ((size_t)blockIdx.x * gridDim.y + blockIdx.y) * vdim;
   const T* gate = gates + (size_t)blockIdx.x * gate_stride + gate_first + (size_t)blockIdx.y * vdim;
   float squares = 0.f;
-  for (int i = threadIdx.x; i < vdim; i += WAVE) squares += read[base + i] * read[base + i];
-  const float scale = rsqrtf(wave_sum(squares) / (float)vdim + eps);
-  for (int i = threadIdx.x; i < vdim; i += WAVE) {
+  __shared__ float shared[17];
+  for (int i = threadIdx.x; i < vdim; i += blockDim.x) squares += read[base + i] * read[base + i];
+  const float scale = rsqrtf((blockDim.x == WAVE ? wave_sum(squares) : block_sum(squares, shared)) / (float)vdim + eps);
+  for (int i = threadIdx.x; i < vdim; i += blockDim.x) {
     const float z = to_float(gate[i]);
-    out[base + i] = from_float<T>(read[base + i] * scale * load_as_float(weight, weight_is_float, i) * (z / (1.f + expf(-z))));
+    const float gated = squash ? 1.f / (1.f + expf(-z)) : z / (1.f + expf(-z));  // sigmoid, or silu
+    out[base + i] = from_float<T>(read[base + i] * scale * load_as_float(weight, weight_is_float, i) * gated);
   }
 }
 
 extern "C" int llmserve_gated_head_norm(const float* read, const void* gates, int is_float, int gate_stride, int gate_first,
                                         const void* weight, int weight_is_float, float eps, int tokens, int heads, int vdim,
-                                        void* out, hipStream_t stream) {
+                                        int squash, void* out, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (heads < 1 || heads > 65535 || vdim < 1 || gate_first + heads * vdim > gate_stride) return ERR_BAD_ARGUMENT;
   const dim3 grid(tokens, heads);
+  const int threads = vdim <= 256 ? WAVE : vdim <= 1024 ? 256 : 512;  // (a norm over all heads at once is one wide "head")
   if (is_float)
-    hipLaunchKernelGGL(gated_head_norm_kernel<float>, grid, dim3(WAVE), 0, stream, read, (const float*)gates, gate_stride, gate_first,
-                       weight, weight_is_float, eps, vdim, (float*)out);
+    hipLaunchKernelGGL(gated_head_norm_kernel<float>, grid, dim3(threads), 0, stream, read, (const float*)gates, gate_stride, gate_first,
+                       weight, weight_is_float, eps, vdim, squash, (float*)out);
   else
-    hipLaunchKernelGGL(gated_head_norm_kernel<bf16_t>, grid, dim3(WAVE), 0, stream, read, (const bf16_t*)gates, gate_stride,
-                       gate_first, weight, weight_is_float, eps, vdim, (bf16_t*)out);
+    hipLaunchKernelGGL(gated_head_norm_kernel<bf16_t>, grid, dim3(threads), 0, stream, read, (const bf16_t*)gates, gate_stride,
+                       gate_first, weight, weight_is_float, eps, vdim, squash, (bf16_t*)out);
   return LAUNCH_STATUS();
 }

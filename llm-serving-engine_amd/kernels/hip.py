@@ -62,9 +62,9 @@ _SIGNATURES = {
     "llmserve_gemm_ring": "pppipiiiiiiip",
     "llmserve_gemm_merged": "ppippipiiiip",
     "llmserve_gemm_tiled": "pppipiiiiiip",
-    "llmserve_attention_generic": "pipipppippiiiiifipfp",
-    "llmserve_attention_f32": "pippppppippiiiiiifiipfp",
-    "llmserve_attention_tiles": "pippppppippiiiiiifiiipippfp",
+    "llmserve_attention_generic": "pipipppippiiiiifipfpp",
+    "llmserve_attention_f32": "pippppppippiiiiiifiipfpp",
+    "llmserve_attention_tiles": "pippppppippiiiiiifiiipippfpp",
     "llmserve_attention_portions": "pippppppippiiiiiifiip",
     "llmserve_attention_can_fuse": "i",
     "llmserve_argmax": "ppppiip",
@@ -87,7 +87,13 @@ _SIGNATURES = {
     "llmserve_causal_conv": "piiiipipppippp",
     "llmserve_gated_delta_rule": "pipppiiiippiiippppp",
     "llmserve_delta_line": "i",
-    "llmserve_gated_head_norm": "ppiiipifiiipp",
+    "llmserve_gated_head_norm": "ppiiipifiiiipp",
+    "llmserve_stream_rows": "ppipiip",
+    "llmserve_add_normed": "ppipipiiifp",
+    "llmserve_assemble_heads": "piiiiiiiiiiiippifpipiifpp",
+    "llmserve_scale_heads": "piiiipiip",
+    "llmserve_soft_cap": "piifp",
+    "llmserve_decay_attention": "piiiiiiiiipppiippp",
 }
 _TYPES = {"p": ctypes.c_void_p, "i": ctypes.c_int, "f": ctypes.c_float}
 
@@ -777,11 +783,12 @@ class HipKernels:
 
     def paged_attention(
         self, qkv, layout, batch, cell, scale: float, window: int | None, *,
-        score_slopes: torch.Tensor | None = None, soft_cap: float | None = None,
+        score_slopes: torch.Tensor | None = None, soft_cap: float | None = None, sinks: torch.Tensor | None = None,
     ) -> torch.Tensor:
         """`score_slopes` (float32 [heads]) and `soft_cap` change the scores before the softmax: cap * tanh(score /
-        cap), then minus slope * distance.  The matrix-core kernels of both precisions take them (in bfloat16
-        not the forms that fuse the rotation or share keys through LDS)."""
+        cap), then minus slope * distance; `sinks` (float32 [heads]) add exp(sink) to a head's denominator.  The
+        matrix-core kernels of both precisions take them (in bfloat16 not the forms that fuse the rotation or share
+        keys through LDS)."""
         tokens = qkv.shape[0]
         group = batch.groups[cell.group]
         if cell.keys.dtype != qkv.dtype:
@@ -790,15 +797,17 @@ class HipKernels:
             raise KernelError("paged_attention: score_slopes is one float32 per query head")
         if soft_cap is not None and not soft_cap > 0:
             raise KernelError("paged_attention: soft_cap must be positive")
+        if sinks is not None and (sinks.dtype != torch.float32 or sinks.shape != (layout.num_heads,)):
+            raise KernelError("paged_attention: sinks is one float32 per query head")
         out = self._empty((tokens, layout.num_heads * layout.head_dim), qkv.dtype)
         dim = layout.head_dim
-        plain_scores = score_slopes is None and soft_cap is None
+        plain_scores = score_slopes is None and soft_cap is None and sinks is None
         if qkv.dtype == torch.bfloat16 and group.page_size % 8 == 0 and dim % 16 == 0 and 16 <= dim <= 256:
-            changed = None if plain_scores else (score_slopes, float(soft_cap or 0.0))
+            changed = None if plain_scores else (score_slopes, float(soft_cap or 0.0), sinks)
             self._attention_tiles(qkv, out, layout, batch, cell, group, scale, int(window or 0), changed=changed)
             return out
         if qkv.dtype == torch.float32 and group.page_size % 4 == 0 and dim % 16 == 0 and 16 <= dim <= 256:
-            self._attention_float32(qkv, out, layout, batch, cell, group, scale, int(window or 0), score_slopes, soft_cap)
+            self._attention_float32(qkv, out, layout, batch, cell, group, scale, int(window or 0), score_slopes, soft_cap, sinks)
             return out
         if qkv.dtype == torch.bfloat16:
             why = f"head size {dim} and pages of {group.page_size}"
@@ -807,12 +816,12 @@ class HipKernels:
             _pointer(qkv), layout.width, _pointer(out), _is_float(qkv), _pointer(cell.keys), _pointer(cell.values),
             _pointer(group.block_tables), group.width, _pointer(batch.token_sequence), _pointer(batch.positions),
             tokens, layout.num_heads, layout.num_kv_heads, dim, group.page_size,
-            scale, int(window or 0), _pointer(score_slopes), float(soft_cap or 0.0), self._stream,
+            scale, int(window or 0), _pointer(score_slopes), float(soft_cap or 0.0), _pointer(sinks), self._stream,
         )
         _check(status, "paged_attention")
         return out
 
-    def _attention_float32(self, qkv, out, layout, batch, cell, group, scale: float, window: int, score_slopes=None, soft_cap=None) -> None:
+    def _attention_float32(self, qkv, out, layout, batch, cell, group, scale: float, window: int, score_slopes=None, soft_cap=None, sinks=None) -> None:
         """The 32-bit path's attention on the matrix cores: an item is 16 (decoding) or 32 columns of one
         request, (token, head) pairs running through the tokens head by head whatever the number of heads; few
         items over long contexts are cut into key splits that a second kernel merges."""
@@ -840,7 +849,7 @@ class HipKernels:
             _pointer(qkv), layout.width, _pointer(out), _pointer(partial_acc), _pointer(partial_ml), _pointer(cell.keys),
             _pointer(cell.values), _pointer(group.block_tables), group.width, _pointer(batch.positions), _pointer(work),
             items, column_tiles, tokens, heads, kv_heads, group.page_size, scale, window, splits, _pointer(score_slopes),
-            float(soft_cap or 0.0), self._stream,
+            float(soft_cap or 0.0), _pointer(sinks), self._stream,
         )
         _check(status, "paged_attention")
 
@@ -851,11 +860,11 @@ class HipKernels:
         store inside the same kernel.  With `unmerged` (a step of single tokens whose reader merges
         key splits itself) the keys are split more finely and the splits are returned as they are
         (their results in bfloat16, laid out for `gemm_merged`; their maxima and sums in float32; how
-        many), instead of `out`.  `changed` = (slopes or None, soft cap or 0.0): scores changed before the softmax,
-        which neither `fuse` nor the kernel that shares keys through LDS takes."""
+        many), instead of `out`.  `changed` = (slopes or None, soft cap or 0.0, sinks or None): scores changed before
+        the softmax or a sink in its denominator, which neither `fuse` nor the kernel that shares keys through LDS takes."""
         if changed is not None and fuse is not None:
             raise KernelError("paged_attention: the fused decode form takes plain scores only")
-        slopes, soft_cap = changed if changed is not None else (None, 0.0)
+        slopes, soft_cap, sinks = changed if changed is not None else (None, 0.0, None)
         library = self._attention_library(layout.head_dim)
         heads, kv_heads = layout.num_heads, layout.num_kv_heads
         per_tile = max(1, 16 // (heads // kv_heads))
@@ -985,7 +994,7 @@ class HipKernels:
                 _pointer(qkv), layout.width, _pointer(out), _pointer(partial_acc), _pointer(partial_ml),
                 _pointer(cell.keys), _pointer(cell.values), _pointer(group.block_tables), group.width, _pointer(batch.positions), _pointer(work), items, column_tiles, tokens, heads, kv_heads,
                 group.page_size, scale, window, splits, (1 if fuse is not None else 0) + (2 if unmerged else 0) + (4 if by_item else 0),
-                _pointer(table), _PAIRINGS[pairing], _pointer(group.slot_mapping), _pointer(slopes), soft_cap, self._stream,
+                _pointer(table), _PAIRINGS[pairing], _pointer(group.slot_mapping), _pointer(slopes), soft_cap, _pointer(sinks), self._stream,
             )
             _check(status, "paged_attention")
             if unmerged and splits > 1:
@@ -1286,7 +1295,7 @@ class HipKernels:
         return out
 
     def gated_head_norm(self, read, gates, gate_first: int, weight, eps: float, heads: int, vdim: int, activation: str) -> torch.Tensor:
-        if activation != "silu":
+        if activation not in ("silu", "sigmoid"):
             raise KernelError(f"gated_head_norm: no kernel gates by {activation!r}")
         tokens = read.shape[0]
         if read.dtype != torch.float32 or read.shape[1] != heads * vdim or weight.shape != (vdim,):
@@ -1294,10 +1303,94 @@ class HipKernels:
         out = self._empty((tokens, heads * vdim), gates.dtype)
         status = self._library_of("delta_rule").llmserve_gated_head_norm(
             _pointer(read), _pointer(gates), _is_float(gates), gates.shape[1], gate_first, _pointer(weight), _is_float(weight), eps,
-            tokens, heads, vdim, _pointer(out), self._stream,
+            tokens, heads, vdim, 1 if activation == "sigmoid" else 0, _pointer(out), self._stream,
         )
         _check(status, "gated_head_norm")
         return out
+
+    # ------------------------------------------------------------------ norms on results, heads put together, linear attention
+
+    def stream_rows(self, hidden, delta) -> torch.Tensor:
+        rows, width = hidden.shape
+        if hidden.dtype != torch.float32 or (delta is not None and delta.dtype != torch.float32):
+            raise KernelError("stream_rows: the residual stream and what is added to it are float32")
+        out = None if self.dtype == torch.float32 else self._empty((rows, width), self.dtype)
+        parts = 1 if delta is None or delta.ndim == 2 else delta.shape[0]
+        status = self._library_of("heads").llmserve_stream_rows(_pointer(hidden), _pointer(delta), parts, _pointer(out), rows, width, self._stream)
+        _check(status, "stream_rows")
+        return hidden if out is None else out
+
+    def add_normed(self, hidden, update, weight, eps: float) -> torch.Tensor:
+        rows, width = hidden.shape
+        if hidden.dtype != torch.float32 or update.dtype != torch.float32 or update.shape[-2:] != (rows, width) or weight.shape != (width,):
+            raise KernelError("add_normed: a float32 stream, float32 rows (or parts of them) of its shape and a weight as long as a row")
+        out = None if self.dtype == torch.float32 else self._empty((rows, width), self.dtype)
+        parts = 1 if update.ndim == 2 else update.shape[0]
+        status = self._library_of("heads").llmserve_add_normed(
+            _pointer(hidden), _pointer(update), parts, _pointer(weight), _is_float(weight), _pointer(out), 0, rows, width, eps, self._stream
+        )
+        _check(status, "add_normed")
+        return hidden if out is None else out
+
+    def assemble_heads(self, x, q_first: int, k_first: int, v_first: int, heads: int, kv_heads: int, dim: int, vdim: int, width: int,
+                       norm, q_weight, k_weight, eps: float, table, rot_dims: int, other=None, other_first: int = 0, blend: float = 0.0):
+        tokens = x.shape[0]
+        if norm not in (None, "head", "row"):
+            raise KernelError(f"assemble_heads: no kernel norms by {norm!r}")
+        if norm is not None:
+            length = dim if norm == "head" else None
+            if q_weight.dtype != k_weight.dtype or q_weight.shape != (length or heads * dim,) or k_weight.shape != (length or kv_heads * dim,):
+                raise KernelError("assemble_heads: the norms' weights are of one type, as long as a head or as the projection")
+        if rot_dims and (table is None or table.dtype != torch.float32 or table.shape != (tokens, rot_dims // 2, 2)):
+            raise KernelError("assemble_heads: a float32 table entry for every pair of every token")
+        if other is not None and (other.dtype != x.dtype or other.shape[0] != tokens):
+            raise KernelError("assemble_heads: the other values are rows of the same type, one a token")
+        out = self._empty((tokens, (heads + 2 * kv_heads) * width), x.dtype)
+        status = self._library_of("heads").llmserve_assemble_heads(
+            _pointer(x), _is_float(x), tokens, x.shape[1], q_first, k_first, v_first, heads, kv_heads, dim, vdim, width,
+            {None: 0, "head": 1, "row": 2}[norm], _pointer(q_weight if norm else None), _pointer(k_weight if norm else None),
+            _is_float(q_weight) if norm else 0, eps, _pointer(table if rot_dims else None), rot_dims, _pointer(other),
+            other.shape[1] if other is not None else 0, other_first, float(blend), _pointer(out), self._stream,
+        )
+        _check(status, "assemble_heads")
+        return out
+
+    def scale_heads(self, x, heads: int, width: int, gates, gate_first: int, squash: str) -> torch.Tensor:
+        if squash != "sigmoid":
+            raise KernelError(f"scale_heads: no kernel squashes a gate by {squash!r}")
+        if x.shape[1] != heads * width or gates.dtype != x.dtype or gates.shape[0] != x.shape[0]:
+            raise KernelError("scale_heads: rows of heads and gates of the same type, a row a token")
+        status = self._library_of("heads").llmserve_scale_heads(
+            _pointer(x), _is_float(x), x.shape[0], heads, width, _pointer(gates), gates.shape[1], gate_first, self._stream
+        )
+        _check(status, "scale_heads")
+        return x
+
+    def decay_attention(self, x, q_first: int, k_first: int, v_first: int, heads: int, dim: int, vdim: int, decays, activation: str,
+                        batch, state) -> torch.Tensor:
+        if activation not in ("silu", "none"):
+            raise KernelError(f"decay_attention: no kernel applies {activation!r} to the projections")
+        tokens = x.shape[0]
+        if state.dtype != torch.float32 or state.shape[1:] != (heads, dim, vdim) or decays.dtype != torch.float32 or decays.shape != (heads,):
+            raise KernelError("decay_attention: a float32 state [slots, heads, dim, vdim] and a float32 decay a head")
+        key = ("decay_attention", dim)
+        if key not in self._lazy:
+            self._lazy[key] = _declared(load_module("decay_attention", {"HEAD_DIM": dim}))
+        out = self._empty((tokens, heads * vdim), torch.float32)
+        status = self._lazy[key].llmserve_decay_attention(
+            _pointer(x), _is_float(x), tokens, x.shape[1], q_first, k_first, v_first, heads, vdim, 1 if activation == "silu" else 0,
+            _pointer(decays), _pointer(batch.query_start), _pointer(batch.state_slots), batch.state_slots.shape[0],
+            int(getattr(batch, "max_query_length", tokens)), _pointer(state), _pointer(out), self._stream,
+        )
+        _check(status, "decay_attention")
+        return out
+
+    def soft_cap(self, logits, cap: float) -> torch.Tensor:
+        if logits.dtype != torch.float32 or logits.ndim != 2:
+            raise KernelError("soft_cap: float32 rows")
+        status = self._library_of("heads").llmserve_soft_cap(_pointer(logits), logits.shape[0], logits.shape[1], float(cap), self._stream)
+        _check(status, "soft_cap")
+        return logits
 
     # ------------------------------------------------------------------ sampling
 

@@ -105,12 +105,13 @@ def window_attention(q, k, v, scale, window, cap=None, sinks=None):
 
 
 def mix_values(v, shared, tensors, prefix):
-    """The first layer that mixes gives its values to the later ones: they take (1 - a) v + a v_first."""
+    """The first layer that mixes gives its values (a token's, all heads side by side) to the later ones: they take
+    (1 - a) v + a v_first."""
     if "first" not in shared:
-        shared["first"] = v
+        shared["first"] = v.reshape(v.shape[0], -1)
         return v
     a = tensors[prefix + "vmix"]
-    return (1.0 - a) * v + a * shared["first"]
+    return (1.0 - a) * v + a * shared["first"].reshape(v.shape)
 
 
 def attention_mixer(h, positions, m, tensors, prefix, eps, shared):
