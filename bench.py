@@ -29,6 +29,10 @@ microseconds and PFLOP/s, counting the causal half only.
 
 measures the engine's second architecture (configs/dafutar-w1536.json, configs/dafutar-w3584.json) beside a Qwen2 of the
 same width, number of layer runs and vocabulary: decoding at --batch and the prefill of --prefill-len tokens.
+
+    python bench.py --op sozavik
+
+does the same for the third (configs/sozavik-w1536.json, configs/sozavik-w3584.json).
 """
 
 from __future__ import annotations
@@ -70,7 +74,7 @@ def parse() -> argparse.Namespace:
                         help="leave out decoding at contexts of 8k and 30k (batch 8) and 4k (batch 64), and the long prompts")
     parser.add_argument("--skip-other-models", action="store_true",
                         help="leave out the float32 run and the 7B and 32B layer sizes")
-    parser.add_argument("--op", choices=("decode-attention", "prefill-attention", "dafutar"), default=None,
+    parser.add_argument("--op", choices=("decode-attention", "prefill-attention", "dafutar", "sozavik"), default=None,
                         help="measure one operation alone instead, as the reference's kernel benchmark does")
     return parser.parse_args()
 
@@ -421,6 +425,8 @@ def main() -> int:
         return prefill_attention_table(args)
     if args.op == "dafutar":
         return dafutar_table(args)
+    if args.op == "sozavik":
+        return sozavik_table(args)
 
     import torch
 
@@ -554,21 +560,32 @@ def dafutar_table(args) -> int:
     two layer sizes beside a Qwen2 of the same width, number of layer runs and vocabulary: decoding at `--batch`
     requests after `--prompt-len`-token prompts and the prefill of a `--prefill-len`-token prompt, random weights.
     One JSON line; the default run of this file is not touched."""
+    return beside_qwen2(args, "dafutar", "Dafutar")
+
+
+def sozavik_table(args) -> int:
+    """The Sozavik decoder (layers of decaying linear attention and of two kinds of normed window attention, norms on the
+    sublayers' results) at two layer sizes beside a Qwen2 of the same width, number of layers, feed-forward and
+    vocabulary, measured as `dafutar_table` measures."""
+    return beside_qwen2(args, "sozavik", "Sozavik")
+
+
+def beside_qwen2(args, name: str, title: str) -> int:
     import torch
 
     pairs = [
-        ("w1536", ROOT / "configs" / "dafutar-w1536.json", ROOT / "configs" / "qwen2-w1536-12-layers.json"),
-        ("w3584", ROOT / "configs" / "dafutar-w3584.json", ROOT / "configs" / "qwen2-w3584-4-layers.json"),
+        ("w1536", ROOT / "configs" / f"{name}-w1536.json", ROOT / "configs" / "qwen2-w1536-12-layers.json"),
+        ("w3584", ROOT / "configs" / f"{name}-w3584.json", ROOT / "configs" / "qwen2-w3584-4-layers.json"),
     ]
     steps, warmup, repeats = max(1, min(args.steps, 64)), min(args.warmup, 8), min(max(1, args.repeats), 3)
     shape = (args.batch, args.prompt_len, output_tokens(args.batch, args.prompt_len, steps, warmup))
     points: dict = {}
     for tag, *paths in pairs:
-        for name, path in zip(("dafutar", "qwen2"), paths):
+        for label, path in zip((name, "qwen2"), paths):
             bench = Bench(str(path), args.dtype, args.seed, library_products=not args.own_products, shapes=[shape], prefill_tokens=args.prefill_len)
             decode = bench.decode(args.batch, args.prompt_len, steps, warmup, repeats)
             prefill = bench.prefill(args.prefill_len, repeats=3)
-            key = f"{name}_{tag}"
+            key = f"{label}_{tag}"
             put(points, f"{key}_decode_b{args.batch}", decode)
             points[f"{key}_prefill"] = prefill["value"]
             points[f"{key}_prefill_ms"] = prefill["ms"]
@@ -579,7 +596,7 @@ def dafutar_table(args) -> int:
             del bench
             torch.cuda.empty_cache()
     print(json.dumps({
-        "metric": f"decode tok/s at batch {args.batch} and prefill tok/s of {args.prefill_len} tokens, Dafutar beside Qwen2 at equal sizes",
+        "metric": f"decode tok/s at batch {args.batch} and prefill tok/s of {args.prefill_len} tokens, {title} beside Qwen2 at equal sizes",
         "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "dtype": args.dtype,
         "data": "synthetic: seeded random weights, uniform random token ids", "points": points,
     }))

@@ -69,6 +69,8 @@ def _read_mixer(kind: str, values: dict[str, Any], where: str):
     if kind == "lightning":
         heads = reader.integer("heads")
         decay = values.get("decay")
+        if isinstance(decay, (int, float)) and not isinstance(decay, bool):  # one number for all heads
+            decay = [decay] * heads
         if not isinstance(decay, list) or len(decay) != heads or any(isinstance(d, bool) or not isinstance(d, (int, float)) for d in decay):
             raise ConfigError(f"{where}: 'decay' must list one number a head")
         return SozavikLightningMixer(heads=heads, dim=reader.integer("dim"), vdim=reader.integer("vdim"), decay=tuple(float(d) for d in decay))
@@ -82,7 +84,7 @@ def _read_mixer(kind: str, values: dict[str, Any], where: str):
             scale_reader = KeyReader(_mapping(values["rot"]["scaling"], f"{where}.rot.scaling"), f"{where}.rot.scaling")
             scaling = tuple(scale_reader.number(name) for name in ("factor", "low", "high", "original"))
         rot = SozavikRotary(found.number("base"), found.integer("dims", minimum=2), scaling)
-        softcap = reader.number("softcap")
+        softcap = reader.number("softcap") if reader.optional("softcap") is not None else None
     return SozavikAttentionMixer(
         heads=heads, kv_heads=reader.integer("kv_heads", default=heads), dim=reader.integer("dim"), vdim=reader.integer("vdim"),
         scale=reader.number("scale"), window=mask.integer("size"), v_mix=reader.boolean("v_mix", default=False), softcap=softcap, rot=rot,

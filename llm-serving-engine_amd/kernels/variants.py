@@ -16,7 +16,7 @@ DEFAULT_VARIANTS: dict[str, list[dict[str, object]]] = {
     "delta_rule": [{}],
     "heads": [{}],
     # query/key sizes of the tests' and the benchmark's models with decaying linear attention
-    "decay_attention": [{"HEAD_DIM": d} for d in (16, 24, 32, 48, 64, 128)],
+    "decay_attention": [{"HEAD_DIM": d} for d in (8, 16, 24, 32, 48, 64, 128)],
     # head sizes of the tests' models and kernel tests, and of the benchmark
     "attention_bf16": [{"HEAD_DIM": d} for d in (16, 32, 48, 64, 80, 96, 112, 128, 144, 160, 192, 256)],
     "attention_f32": [{"HEAD_DIM": d} for d in (16, 32, 48, 64, 80, 96, 112, 128, 144, 160, 192, 256)],

@@ -52,7 +52,7 @@ def test_config_round_trip_and_refusals():
         cases.config_of([(cases.attention(), {"kind": "sparse", "ff": 8})]),
     ]
     missing = cases.config_of([(cases.attention(), None)])
-    del missing["layers"][0]["mixer"]["softcap"]
+    del missing["layers"][0]["mixer"]["scale"]
     for values in broken + [missing, {**cases.MIXED, "width": None}]:
         with pytest.raises(ConfigError):
             SozavikConfig.from_dict(values)
