@@ -93,7 +93,7 @@ _SIGNATURES = {
     "llmserve_assemble_heads": "piiiiiiiiiiiippifpipiifpp",
     "llmserve_scale_heads": "piiiipiip",
     "llmserve_soft_cap": "piifp",
-    "llmserve_decay_attention": "piiiiiiiiipppiippp",
+    "llmserve_decay_attention": "piiiiiiiiipppiippiipp",
 }
 _TYPES = {"p": ctypes.c_void_p, "i": ctypes.c_int, "f": ctypes.c_float}
 
@@ -1377,10 +1377,20 @@ class HipKernels:
         if key not in self._lazy:
             self._lazy[key] = _declared(load_module("decay_attention", {"HEAD_DIM": dim}))
         out = self._empty((tokens, heads * vdim), torch.float32)
+        requests, longest = batch.state_slots.shape[0], int(getattr(batch, "max_query_length", tokens))
+        # A long portion is walked in segments side by side (a walk is a chain of runs of 16 tokens, one after the other):
+        # segments of 128 tokens from 256 tokens on, longer ones where there would be more than 64 of them.
+        segment = 128
+        while longest > 64 * segment:
+            segment *= 2
+        segments = -(-longest // segment) if longest >= 256 else 1
+        if segments == 1:
+            segment = -(-max(longest, 16) // 16) * 16
+        carry = self._empty((requests * segments, heads, dim, vdim), torch.float32) if segments > 1 else None
         status = self._lazy[key].llmserve_decay_attention(
             _pointer(x), _is_float(x), tokens, x.shape[1], q_first, k_first, v_first, heads, vdim, 1 if activation == "silu" else 0,
-            _pointer(decays), _pointer(batch.query_start), _pointer(batch.state_slots), batch.state_slots.shape[0],
-            int(getattr(batch, "max_query_length", tokens)), _pointer(state), _pointer(out), self._stream,
+            _pointer(decays), _pointer(batch.query_start), _pointer(batch.state_slots), requests, longest, _pointer(state),
+            _pointer(out), segment, segments, _pointer(carry), self._stream,
         )
         _check(status, "decay_attention")
         return out

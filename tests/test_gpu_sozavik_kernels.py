@@ -109,10 +109,11 @@ def test_gated_head_norm_wide_and_squashed(kernels, dtype, activation, heads, vd
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,dim,vdim", [(3, 32, 48), (2, 16, 16), (2, 24, 40), (1, 48, 70), (2, 64, 128)])
-@pytest.mark.parametrize("counts", [[1, 1, 1], [37, 1, 16], [2, 3, 1], [17, 64, 5]])
+@pytest.mark.parametrize("counts", [[1, 1, 1], [37, 1, 16], [2, 3, 1], [17, 64, 5], [300, 1, 530], [256, 129, 128]])
 def test_decay_attention(kernels, dtype, heads, dim, vdim, counts):
     """Steps of single tokens, of runs that end anywhere, and of both; states carried over; both kernels (sizes that
-    are multiples of 16 walk runs on the matrix cores where a request brings four tokens or more)."""
+    are multiples of 16 walk runs on the matrix cores where a request brings four tokens or more, in segments side by
+    side where one brings 256 or more)."""
     torch.manual_seed(dim + vdim + sum(counts))
     tokens = sum(counts)
     row = 5 + 2 * heads * dim + heads * vdim  # (the columns begin where 16-byte loads may not: the kernels decide by that)
