@@ -43,6 +43,34 @@ extern "C" int llmserve_stream_rows(float* hidden, const float* delta, int parts
 // cut over K, added in order).  One block per row; a row whose length is a multiple of 4 stays in registers in
 // 16-byte pieces, and all of a thread's loads are asked for before the first is used.  The sum of squares is added
 // in an order that depends only on the row length.  `out` (run dtype) gets the new row, or is null.
+template <int PARTS, int PIECES>
+__device__ __forceinline__ void add_parts(float4 (&v)[PIECES], const float* from, size_t part_stride, int quads) {
+#pragma unroll
+  for (int j = 0; j < PIECES; ++j) {
+    const int i = min((int)(threadIdx.x + j * blockDim.x), quads - 1);
+    float4 d[PARTS];
+#pragma unroll
+    for (int p = 0; p < PARTS; ++p) d[p] = ((const float4*)(from + (size_t)p * part_stride))[i];
+#pragma unroll
+    for (int p = 0; p < PARTS; ++p) {
+      v[j].x += d[p].x; v[j].y += d[p].y; v[j].z += d[p].z; v[j].w += d[p].w;
+    }
+  }
+}
+
+template <int PIECES>
+__device__ __forceinline__ void add_some_parts(float4 (&v)[PIECES], const float* from, int count, size_t part_stride, int quads) {
+  switch (count) {
+    case 1: add_parts<1, PIECES>(v, from, part_stride, quads); break;
+    case 2: add_parts<2, PIECES>(v, from, part_stride, quads); break;
+    case 3: add_parts<3, PIECES>(v, from, part_stride, quads); break;
+    case 4: add_parts<4, PIECES>(v, from, part_stride, quads); break;
+    case 5: add_parts<5, PIECES>(v, from, part_stride, quads); break;
+    case 6: add_parts<6, PIECES>(v, from, part_stride, quads); break;
+    default: add_parts<7, PIECES>(v, from, part_stride, quads); break;
+  }
+}
+
 template <typename TO, int PIECES>
 __global__ __launch_bounds__(1024) void add_normed_vector_kernel(float* __restrict__ hidden, const float* __restrict__ update,
                                                                  int parts, size_t part_stride, const void* __restrict__ weight,
@@ -63,14 +91,9 @@ __global__ __launch_bounds__(1024) void add_normed_vector_kernel(float* __restri
     else
       narrow[j] = ((const uint2*)weight)[i];
   }
-  for (int p = 1; p < parts; ++p) {
-#pragma unroll
-    for (int j = 0; j < PIECES; ++j) {
-      const int i = min((int)(threadIdx.x + j * blockDim.x), quads - 1);
-      const float4 d = ((const float4*)(from + (size_t)p * part_stride))[i];
-      u[j].x += d.x; u[j].y += d.y; u[j].z += d.z; u[j].w += d.w;
-    }
-  }
+  // the further parts are added in order, up to seven at a time: their loads are all asked for before the first is used
+  for (int first = 1; first < parts; first += 7)
+    add_some_parts<PIECES>(u, from + (size_t)first * part_stride, min(parts - first, 7), part_stride, quads);
   float squares = 0.f;
 #pragma unroll
   for (int j = 0; j < PIECES; ++j)
@@ -155,16 +178,18 @@ extern "C" int llmserve_add_normed(float* hidden, const float* update, int parts
 // weight of `dim` shared by the heads; 2: all heads of the projection together, the weight as long as they; 0: not),
 // its first `rot_dims` dimensions are turned in pairs (2i, 2i + 1) by (cos, sin) of table[token][i], and it is written
 // `width` wide, zeros beyond `dim`.  A value head of `vdim` is blended with the same columns of `other` and written
-// `width` wide.  The output row is [heads | kv_heads | kv_heads] heads of `width`.
+// `width` wide.  The output row is [heads | kv_heads | kv_heads] heads of `width`; the keys and values may go to
+// their pages in the same kernel (a step of single tokens: one launch less).
 struct HeadSizes {
   int x_width, q_first, k_first, v_first, heads, kv_heads, dim, vdim, width, norm, rot_dims, other_width, other_first;
 };
 
 template <typename T>
-__global__ __launch_bounds__(256) void assemble_heads_kernel(const T* __restrict__ x, HeadSizes z, const void* __restrict__ q_weight,
-                                                             const void* __restrict__ k_weight, int weight_is_float, float eps,
-                                                             const float* __restrict__ table, const T* __restrict__ other,
-                                                             float blend, T* __restrict__ out) {
+__global__ __launch_bounds__(1024) void assemble_heads_kernel(const T* __restrict__ x, HeadSizes z, const void* __restrict__ q_weight,
+                                                              const void* __restrict__ k_weight, int weight_is_float, float eps,
+                                                              const float* __restrict__ table, const T* __restrict__ other,
+                                                              float blend, T* __restrict__ out, T* __restrict__ keys,
+                                                              T* __restrict__ values, const int* __restrict__ slots, int page_size) {
   __shared__ float shared[17];
   const size_t token = blockIdx.x;
   const T* row = x + token * z.x_width;
@@ -217,17 +242,32 @@ __global__ __launch_bounds__(256) void assemble_heads_kernel(const T* __restrict
       dst[(size_t)unit * z.width + e] = from_float<T>(result);
     }
   }
-  const T* values = row + z.v_first;
+  const T* own = row + z.v_first;
   const T* given = other ? other + token * z.other_width + z.other_first : nullptr;
   T* value_dst = dst + (size_t)(z.heads + z.kv_heads) * z.width;
   for (int index = threadIdx.x; index < z.kv_heads * z.width; index += blockDim.x) {
     const int head = index / z.width, e = index % z.width;
     float result = 0.f;
     if (e < z.vdim) {
-      result = to_float(values[head * z.vdim + e]);
+      result = to_float(own[head * z.vdim + e]);
       if (given) result = (1.f - blend) * result + blend * to_float(given[head * z.vdim + e]);
     }
     value_dst[index] = from_float<T>(result);
+  }
+  // With `slots` (page * page_size + offset of every token, negative: nowhere) the token's keys and values also go
+  // to its place in the pages, read back from the row just written.
+  if (slots == nullptr) return;
+  const int slot = slots[token];
+  if (slot < 0) return;
+  __syncthreads();
+  const int page = slot / page_size, offset = slot % page_size;
+  const T* k_row = dst + (size_t)z.heads * z.width;
+  const T* v_row = k_row + (size_t)z.kv_heads * z.width;
+  for (int index = threadIdx.x; index < z.kv_heads * z.width; index += blockDim.x) {
+    const int head = index / z.width, d = index % z.width;
+    const size_t block = ((size_t)page * z.kv_heads + head) * page_size * z.width;
+    keys[block + key_element(d, offset, page_size, z.width)] = k_row[index];
+    values[block + value_element(d, offset, page_size, z.width)] = v_row[index];
   }
 }
 
@@ -235,7 +275,7 @@ extern "C" int llmserve_assemble_heads(const void* x, int is_float, int tokens, 
                                        int heads, int kv_heads, int dim, int vdim, int width, int norm, const void* q_weight,
                                        const void* k_weight, int weight_is_float, float eps, const float* table, int rot_dims,
                                        const void* other, int other_width, int other_first, float blend, void* out,
-                                       hipStream_t stream) {
+                                       void* keys, void* values, const int* slots, int page_size, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (heads < 1 || kv_heads < 1 || dim < 1 || vdim < 1 || width < dim || width < vdim || norm < 0 || norm > 2 ||
       (norm && (!q_weight || !k_weight)) || rot_dims < 0 || rot_dims % 2 || rot_dims > dim || (rot_dims && !table) ||
@@ -243,12 +283,17 @@ extern "C" int llmserve_assemble_heads(const void* x, int is_float, int tokens, 
       v_first + kv_heads * vdim > x_width || (other && (other_first < 0 || other_first + kv_heads * vdim > other_width)))
     return ERR_BAD_ARGUMENT;
   const HeadSizes z = {x_width, q_first, k_first, v_first, heads, kv_heads, dim, vdim, width, norm, rot_dims, other_width, other_first};
+  if (slots && (!keys || !values || page_size < 1)) return ERR_BAD_ARGUMENT;
+  // a wave a head where there are up to sixteen of them (a step of few tokens is as long as its longest workgroup)
+  const int threads = WAVE * max(4, min(16, heads + kv_heads));
   if (is_float)
-    hipLaunchKernelGGL(assemble_heads_kernel<float>, dim3(tokens), dim3(256), 0, stream, (const float*)x, z, q_weight, k_weight,
-                       weight_is_float, eps, table, (const float*)other, blend, (float*)out);
+    hipLaunchKernelGGL(assemble_heads_kernel<float>, dim3(tokens), dim3(threads), 0, stream, (const float*)x, z, q_weight, k_weight,
+                       weight_is_float, eps, table, (const float*)other, blend, (float*)out, (float*)keys, (float*)values, slots,
+                       page_size);
   else
-    hipLaunchKernelGGL(assemble_heads_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream, (const bf16_t*)x, z, q_weight, k_weight,
-                       weight_is_float, eps, table, (const bf16_t*)other, blend, (bf16_t*)out);
+    hipLaunchKernelGGL(assemble_heads_kernel<bf16_t>, dim3(tokens), dim3(threads), 0, stream, (const bf16_t*)x, z, q_weight, k_weight,
+                       weight_is_float, eps, table, (const bf16_t*)other, blend, (bf16_t*)out, (bf16_t*)keys, (bf16_t*)values, slots,
+                       page_size);
   return LAUNCH_STATUS();
 }
 

@@ -90,7 +90,7 @@ _SIGNATURES = {
     "llmserve_gated_head_norm": "ppiiipifiiiipp",
     "llmserve_stream_rows": "ppipiip",
     "llmserve_add_normed": "ppipipiiifp",
-    "llmserve_assemble_heads": "piiiiiiiiiiiippifpipiifpp",
+    "llmserve_assemble_heads": "piiiiiiiiiiiippifpipiifppppip",
     "llmserve_scale_heads": "piiiipiip",
     "llmserve_soft_cap": "piifp",
     "llmserve_decay_attention": "piiiiiiiiipppiippiipp",
@@ -1333,7 +1333,10 @@ class HipKernels:
         return hidden if out is None else out
 
     def assemble_heads(self, x, q_first: int, k_first: int, v_first: int, heads: int, kv_heads: int, dim: int, vdim: int, width: int,
-                       norm, q_weight, k_weight, eps: float, table, rot_dims: int, other=None, other_first: int = 0, blend: float = 0.0):
+                       norm, q_weight, k_weight, eps: float, table, rot_dims: int, other=None, other_first: int = 0, blend: float = 0.0,
+                       batch=None, cell=None):
+        """With a writable `cell` the keys and values are also stored in its pages: by this kernel in a step of single
+        tokens, by the kernel that stores prompt portions (whole pieces of a page at a time) otherwise."""
         tokens = x.shape[0]
         if norm not in (None, "head", "row"):
             raise KernelError(f"assemble_heads: no kernel norms by {norm!r}")
@@ -1346,13 +1349,25 @@ class HipKernels:
         if other is not None and (other.dtype != x.dtype or other.shape[0] != tokens):
             raise KernelError("assemble_heads: the other values are rows of the same type, one a token")
         out = self._empty((tokens, (heads + 2 * kv_heads) * width), x.dtype)
+        store = cell is not None and cell.writable
+        group = batch.groups[cell.group] if store else None
+        if store and (cell.keys.dtype != x.dtype or cell.values.shape[1:] != cell.need.page_fields(group.page_size)["values"]
+                      or (cell.need.num_kv_heads, cell.need.head_dim) != (kv_heads, width)):
+            raise KernelError("assemble_heads: the cell's pages do not fit the heads")
+        here = store and batch.max_query_length == 1
         status = self._library_of("heads").llmserve_assemble_heads(
             _pointer(x), _is_float(x), tokens, x.shape[1], q_first, k_first, v_first, heads, kv_heads, dim, vdim, width,
             {None: 0, "head": 1, "row": 2}[norm], _pointer(q_weight if norm else None), _pointer(k_weight if norm else None),
             _is_float(q_weight) if norm else 0, eps, _pointer(table if rot_dims else None), rot_dims, _pointer(other),
-            other.shape[1] if other is not None else 0, other_first, float(blend), _pointer(out), self._stream,
+            other.shape[1] if other is not None else 0, other_first, float(blend), _pointer(out),
+            _pointer(cell.keys if here else None), _pointer(cell.values if here else None), _pointer(group.slot_mapping if here else None),
+            group.page_size if here else 1, self._stream,
         )
         _check(status, "assemble_heads")
+        if store and not here:
+            from ..parts.position import HeadLayout
+
+            self.rotate_and_store(out, HeadLayout(heads, kv_heads, width), batch, cell, None, "none")
         return out
 
     def scale_heads(self, x, heads: int, width: int, gates, gate_first: int, squash: str) -> torch.Tensor:

@@ -161,13 +161,16 @@ class Kernels(Protocol):
         self, x: torch.Tensor, q_first: int, k_first: int, v_first: int, heads: int, kv_heads: int, dim: int, vdim: int,
         width: int, norm: str | None, q_weight: torch.Tensor | None, k_weight: torch.Tensor | None, eps: float,
         table: torch.Tensor | None, rot_dims: int, other: torch.Tensor | None = None, other_first: int = 0, blend: float = 0.0,
+        batch: Any = None, cell: Any = None,
     ) -> torch.Tensor:
         """From rows that hold `heads` queries and `kv_heads` keys of `dim` and `kv_heads` values of `vdim` (from the
         columns q_first, k_first, v_first): rows [T, (heads + 2 kv_heads) * width] of queries, keys and values of
         `width`, zeros beyond a head's own size.  Queries and keys are RMS-normed (`norm` "head": every head by
         itself, weights of dim; "row": all query heads together and all key heads together, weights as long as
         they; None), then their first `rot_dims` dimensions turned in adjacent pairs by the token's row of `table`
-        (float32 [T, rot_dims / 2, 2], cos and sin).  With `other`: v <- (1 - blend) v + blend * other[:, other_first : + kv_heads * vdim]."""
+        (float32 [T, rot_dims / 2, 2], cos and sin).  With `other`: v <- (1 - blend) v + blend * other[:, other_first : + kv_heads * vdim].
+        With a writable `cell` (and the step's `batch`) the keys and values are also stored in the cell's pages, as
+        `rotate_and_store` without a rotation would store them."""
 
     def scale_heads(self, x: torch.Tensor, heads: int, width: int, gates: torch.Tensor, gate_first: int, squash: str) -> torch.Tensor:
         """x[:, h * width : (h + 1) * width] *= squash(gates[:, gate_first + h]) for every head, in place."""

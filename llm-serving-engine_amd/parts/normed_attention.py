@@ -139,14 +139,15 @@ class NormedAttention(Mixer):
                 raise RuntimeError("normed attention: no earlier layer of this step gave values of this size")
         table = kernels.rotary_table(batch, self.frequencies, self.magnitude) if spec.rot_dims else None
         # per token the heads' queries, keys and values as the attention reads them: normed, turned, blended, widened
+        plain = spec.soft_cap is None and self.sinks is None and not spec.gate
         rows = kernels.assemble_heads(
             projected, 0, q_size, q_size + k_size, spec.num_heads, spec.num_kv_heads, spec.dim, spec.vdim, spec.head_width,
             spec.norm, self.q_norm, self.k_norm, spec.eps, table, spec.rot_dims,
             given[0] if given else None, given[1] if given else 0, self.blend,
+            batch=batch, cell=None if plain else cell,  # (with plain scores the attention below stores, and may fuse that)
         )
-        if spec.soft_cap is None and self.sinks is None and not spec.gate:
+        if plain:
             return kernels.rotate_store_attend(rows, self.layout, batch, cell, None, "none", spec.scale, spec.window, project=self.out)
-        kernels.rotate_and_store(rows, self.layout, batch, cell, None, "none")
         mixed = kernels.paged_attention(rows, self.layout, batch, cell, spec.scale, spec.window, soft_cap=spec.soft_cap, sinks=self.sinks)
         if spec.gate:
             kernels.scale_heads(mixed, spec.num_heads, spec.head_width, projected, q_size + k_size + v_size, "sigmoid")

@@ -171,3 +171,36 @@ def test_attention_with_sinks_and_capped_scores(kernels, dtype, heads, kv_heads,
         want = TorchKernels(dtype).paged_attention(qkv, layout, batch_on("cpu"), plain_cell, 0.2, window, soft_cap=cap, sinks=sinks)
         got = kernels[dtype].paged_attention(gpu(qkv), layout, batch_on("cuda"), device_cell, 0.2, window, soft_cap=cap, sinks=gpu(sinks))
         close(got, want, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("counts", [[1, 1, 1, 1], [5, 1, 9]])
+def test_assemble_heads_stores_keys_and_values(kernels, dtype, counts):
+    """A step of single tokens stores in the kernel that puts the heads together, a step of portions in the kernel that
+    stores portions: the pages hold the same either way, and only at the step's places."""
+    from llmserve_amd.cache.cell import CacheCell
+    from llmserve_amd.parts import PagedKeyValue
+
+    torch.manual_seed(sum(counts))
+    heads, kv_heads, dim, vdim, width, page = 6, 2, 24, 40, 48, 8
+    need = PagedKeyValue(kv_heads, width, None)
+    tokens = sum(counts)
+    fields = {name: torch.randn(12, *shape).to(dtype) for name, shape in need.page_fields(page).items()}
+    slots = torch.randperm(12 * page)[:tokens].to(torch.int32)
+    x = torch.randn(tokens, heads * dim + kv_heads * (dim + vdim)).to(dtype)
+    weight = (1 + 0.3 * torch.randn(dim)).to(dtype)
+
+    def run(library, device):
+        batch = step_of(counts, [3] * len(counts), list(range(len(counts))), device)
+        batch.groups = [types.SimpleNamespace(page_size=page, block_tables=None, slot_mapping=slots.to(device), width=0)]
+        cell = CacheCell(need, group=0, fields={name: value.clone().to(device) for name, value in fields.items()})
+        move = (lambda t: t.to(device))
+        rows = library.assemble_heads(move(x), 0, heads * dim, (heads + kv_heads) * dim, heads, kv_heads, dim, vdim, width, "head",
+                                      move(weight), move(weight), 1e-5, None, 0, batch=batch, cell=cell)
+        return rows, cell
+
+    want_rows, want_cell = run(TorchKernels(dtype), "cpu")
+    got_rows, got_cell = run(kernels[dtype], "cuda")
+    close(got_rows, want_rows, dtype)
+    for name in fields:
+        close(got_cell.fields[name], want_cell.fields[name], dtype)

@@ -280,7 +280,7 @@ class TorchKernels:
         return hidden if self.dtype == torch.float32 else hidden.to(self.dtype)
 
     def assemble_heads(self, x, q_first, k_first, v_first, heads, kv_heads, dim, vdim, width, norm, q_weight, k_weight, eps,
-                       table, rot_dims, other=None, other_first=0, blend=0.0):
+                       table, rot_dims, other=None, other_first=0, blend=0.0, batch=None, cell=None):
         tokens = x.shape[0]
         out = torch.zeros((tokens, heads + 2 * kv_heads, width))
 
@@ -306,7 +306,12 @@ class TorchKernels:
         if other is not None:
             values = (1.0 - blend) * values + blend * other[:, other_first : other_first + kv_heads * vdim].float()
         out[:, heads + kv_heads :, :vdim] = values.reshape(tokens, kv_heads, vdim)
-        return out.reshape(tokens, -1).to(self.dtype)
+        out = out.reshape(tokens, -1).to(self.dtype)
+        if cell is not None and cell.writable:
+            from llmserve_amd.parts import HeadLayout
+
+            self.rotate_and_store(out, HeadLayout(heads, kv_heads, width), batch, cell, None, "none")
+        return out
 
     def scale_heads(self, x, heads, width, gates, gate_first, squash):
         assert squash == "sigmoid"
