@@ -69,13 +69,15 @@ __device__ __forceinline__ double whole_power(double base, int n) {
 }
 
 // What a lane holds of a run of up to 16 tokens, as loaded (not yet activated): Q and K by rows (lane (i, g): d = 16
-// tile + 4 g .. + 3 of token i), and V and K read across (lane (i, g): column i of tokens 4 g + e).
+// tile + 4 g .. + 3 of token i), and V (of each of the wave's VT tiles of 16 columns) and K read across (lane (i, g):
+// column i of tokens 4 g + e).
+template <int VT>
 struct RunOperands {
-  f32x4 q[D_TILES], k[D_TILES], across[D_TILES], v;
+  f32x4 q[D_TILES], k[D_TILES], across[D_TILES], v[VT];
 };
 
-template <typename T>
-__device__ __forceinline__ void load_run(RunOperands& r, const T* __restrict__ x, const DecaySizes& z, int head, int v0, int t0,
+template <typename T, int VT>
+__device__ __forceinline__ void load_run(RunOperands<VT>& r, const T* __restrict__ x, const DecaySizes& z, int head, int v0, int t0,
                                          int n, int i, int g) {
   const T* mine = x + (size_t)(t0 + min(i, n - 1)) * z.x_width + head * D + 4 * g;
 #pragma unroll
@@ -86,18 +88,20 @@ __device__ __forceinline__ void load_run(RunOperands& r, const T* __restrict__ x
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     const T* theirs = x + (size_t)(t0 + min(4 * g + e, n - 1)) * z.x_width;
-    r.v[e] = to_float(theirs[z.v_first + head * z.vdim + v0 + i]);
+#pragma unroll
+    for (int j = 0; j < VT; ++j) r.v[j][e] = to_float(theirs[z.v_first + head * z.vdim + v0 + 16 * j + i]);
 #pragma unroll
     for (int tile = 0; tile < D_TILES; ++tile) r.across[tile][e] = to_float(theirs[z.k_first + head * D + 16 * tile + i]);
   }
 }
 
-// grid (vdim / 16, heads, requests * segments), one wave a workgroup.  A request's tokens are cut into segments of
-// `segment` tokens (a multiple of 16) that are walked side by side: the first starts from the request's state, the
-// others from nothing, and each leaves the state it ends with in `carry` [requests * segments, heads, D, vdim]; the
-// two kernels below then hand the states on and add what a segment's tokens read of the state they start from.
-// With one segment (`carry` null) the state is read and written here and nothing follows.
-template <typename T, bool SILU>
+// grid (vdim / (16 VT), heads, requests * segments), one wave a workgroup, which owns VT tiles of 16 value columns:
+// Q, K and the scores are loaded, activated and computed once for all of them.  A request's tokens are cut into
+// segments of `segment` tokens (a multiple of 16) that are walked side by side: the first starts from the request's
+// state, the others from nothing, and each leaves the state it ends with in `carry` [requests * segments, heads, D,
+// vdim]; the two kernels below then hand the states on and add what a segment's tokens read of the state they start
+// from.  With one segment (`carry` null) the state is read and written here and nothing follows.
+template <typename T, bool SILU, int VT>
 __global__ __launch_bounds__(64) void decay_attention_runs_kernel(const T* __restrict__ x, DecaySizes z,
                                                                   const float* __restrict__ decays,
                                                                   const int* __restrict__ query_start,
@@ -105,26 +109,28 @@ __global__ __launch_bounds__(64) void decay_attention_runs_kernel(const T* __res
                                                                   float* __restrict__ out, int segment, int segments,
                                                                   float* __restrict__ carry) {
   __shared__ float power[RUN + 1];
-  const int v0 = blockIdx.x * 16, head = blockIdx.y, request = blockIdx.z / segments, part = blockIdx.z % segments;
+  const int v0 = blockIdx.x * 16 * VT, head = blockIdx.y, request = blockIdx.z / segments, part = blockIdx.z % segments;
   const int lane = threadIdx.x, i = lane & 15, g = lane >> 4;
   const int begin = query_start[request] + part * segment, end = min(query_start[request + 1], begin + segment);
   if (begin >= end) return;  // a request that only pads a captured step, or one with fewer segments
   if (lane <= RUN) power[lane] = (float)whole_power((double)decays[head], lane);
   __syncthreads();
-  // S[d][v] of this wave's columns: lane (i, g) holds rows 16 tile + 4 g + e of column v0 + i
+  // S[d][v] of this wave's columns: lane (i, g) holds rows 16 tile + 4 g + e of columns v0 + 16 j + i
   float* s_at = state + (((size_t)state_slots[request] * z.heads + head) * D + 4 * g) * z.vdim + v0 + i;
-  f32x4 S[D_TILES];
+  f32x4 S[VT][D_TILES];
 #pragma unroll
-  for (int tile = 0; tile < D_TILES; ++tile)
+  for (int j = 0; j < VT; ++j)
 #pragma unroll
-    for (int e = 0; e < 4; ++e) S[tile][e] = part == 0 ? s_at[(size_t)(16 * tile + e) * z.vdim] : 0.f;
+    for (int tile = 0; tile < D_TILES; ++tile)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) S[j][tile][e] = part == 0 ? s_at[(size_t)(16 * tile + e) * z.vdim + 16 * j] : 0.f;
   const int out_width = z.heads * z.vdim;
 
-  RunOperands next;
+  RunOperands<VT> next;
   load_run(next, x, z, head, v0, begin, min(RUN, end - begin), i, g);
   for (int t0 = begin; t0 < end; t0 += RUN) {
     const int n = min(RUN, end - t0);
-    RunOperands now = next;
+    RunOperands<VT> now = next;
     // The next run's operands are on their way while this run is computed.  (No branch around the loads: a wave waits at
     // a branch's end for what was asked for inside it.  After the last run, that run is asked for again and not used.)
     const int ahead = t0 + RUN < end ? t0 + RUN : t0;
@@ -140,7 +146,8 @@ __global__ __launch_bounds__(64) void decay_attention_runs_kernel(const T* __res
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int s = 4 * g + e;
-      now.v[e] = s < n ? activated_fast<SILU>(now.v[e]) : 0.f;
+#pragma unroll
+      for (int j = 0; j < VT; ++j) now.v[j][e] = s < n ? activated_fast<SILU>(now.v[j][e]) : 0.f;
       const float fade = s < n ? power[n - 1 - s] : 0.f;
 #pragma unroll
       for (int tile = 0; tile < D_TILES; ++tile) now.across[tile][e] = s < n ? activated_fast<SILU>(now.across[tile][e]) * fade : 0.f;
@@ -156,34 +163,44 @@ __global__ __launch_bounds__(64) void decay_attention_runs_kernel(const T* __res
       const int s = 4 * g + e;
       p[e] = s <= i ? p[e] * power[i - s] : 0.f;
     }
-    // O[t][v] = sum_s P[t][s] V[s][v] + sum_d decay^(t+1) Q[t][d] S[d][v]
-    f32x4 o = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int e = 0; e < 4; ++e) o = __builtin_amdgcn_mfma_f32_16x16x4f32(p[e], now.v[e], o, 0, 0, 0);
     const float carried = power[i + 1];
 #pragma unroll
     for (int tile = 0; tile < D_TILES; ++tile)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) o = __builtin_amdgcn_mfma_f32_16x16x4f32(now.q[tile][e] * carried, S[tile][e], o, 0, 0, 0);
-    // S = decay^n S + sum_s decay^(n-1-s) k_s v_s^T
+      for (int e = 0; e < 4; ++e) now.q[tile][e] *= carried;
     const float whole = power[n];
 #pragma unroll
-    for (int tile = 0; tile < D_TILES; ++tile) {
+    for (int j = 0; j < VT; ++j) {
+      // O[t][v] = sum_s P[t][s] V[s][v] + sum_d decay^(t+1) Q[t][d] S[d][v]
+      f32x4 o = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int e = 0; e < 4; ++e) S[tile][e] *= whole;
+      for (int e = 0; e < 4; ++e) o = __builtin_amdgcn_mfma_f32_16x16x4f32(p[e], now.v[j][e], o, 0, 0, 0);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) S[tile] = __builtin_amdgcn_mfma_f32_16x16x4f32(now.across[tile][e], now.v[e], S[tile], 0, 0, 0);
+      for (int tile = 0; tile < D_TILES; ++tile)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o = __builtin_amdgcn_mfma_f32_16x16x4f32(now.q[tile][e], S[j][tile][e], o, 0, 0, 0);
+      // S = decay^n S + sum_s decay^(n-1-s) k_s v_s^T
+#pragma unroll
+      for (int tile = 0; tile < D_TILES; ++tile) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) S[j][tile][e] *= whole;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          S[j][tile] = __builtin_amdgcn_mfma_f32_16x16x4f32(now.across[tile][e], now.v[j][e], S[j][tile], 0, 0, 0);
+      }
+      // lane (i, g) holds O[t = 4 g + e][v0 + 16 j + i]
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (4 * g + e < n) out[(size_t)(t0 + 4 * g + e) * out_width + head * z.vdim + v0 + 16 * j + i] = o[e];
     }
-    // lane (i, g) holds O[t = 4 g + e][v0 + i]
-#pragma unroll
-    for (int e = 0; e < 4; ++e)
-      if (4 * g + e < n) out[(size_t)(t0 + 4 * g + e) * out_width + head * z.vdim + v0 + i] = o[e];
   }
   float* left = carry ? carry + (((size_t)blockIdx.z * z.heads + head) * D + 4 * g) * z.vdim + v0 + i : s_at;
 #pragma unroll
-  for (int tile = 0; tile < D_TILES; ++tile)
+  for (int j = 0; j < VT; ++j)
 #pragma unroll
-    for (int e = 0; e < 4; ++e) left[(size_t)(16 * tile + e) * z.vdim] = S[tile][e];
+    for (int tile = 0; tile < D_TILES; ++tile)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) left[(size_t)(16 * tile + e) * z.vdim + 16 * j] = S[j][tile][e];
 }
 
 // The states handed on from segment to segment, one thread an element of S: what segment j left, F_j = decay^(its
@@ -357,8 +374,14 @@ extern "C" int llmserve_decay_attention(const void* x, int is_float, int tokens,
     if (segments < 1 || segment < RUN || segment % RUN || (segments > 1 && !carry) || (long)requests * segments > 65535 ||
         (long)segment * segments < longest)
       return ERR_BAD_ARGUMENT;
-    const dim3 grid(vdim / 16, heads, requests * segments);
     float* kept = segments > 1 ? carry : nullptr;
+    // How many tiles of 16 value columns a wave owns: what it loads and activates of Q and K serves them all, so as many
+    // (1, 2 or 4; one where S's rows alone fill the registers) as still leave a wave for three SIMDs in four.
+    const long tiles = (long)(vdim / 16) * heads * requests * segments;
+    const int most = D <= 128 ? 4 : 1;
+    int owned = 1;
+    while (owned < most && vdim % (32 * owned) == 0 && tiles / (2 * owned) >= 768) owned *= 2;
+    dim3 grid(vdim / (16 * owned), heads, requests * segments);
 #define LAUNCH_RUNS(KERNEL, ...)                                                                                                 \
   do {                                                                                                                          \
     if (is_float && activation) hipLaunchKernelGGL((KERNEL<float, true>), grid, dim3(64), 0, stream, (const float*)x, __VA_ARGS__);   \
@@ -366,7 +389,18 @@ extern "C" int llmserve_decay_attention(const void* x, int is_float, int tokens,
     else if (activation) hipLaunchKernelGGL((KERNEL<bf16_t, true>), grid, dim3(64), 0, stream, (const bf16_t*)x, __VA_ARGS__);      \
     else hipLaunchKernelGGL((KERNEL<bf16_t, false>), grid, dim3(64), 0, stream, (const bf16_t*)x, __VA_ARGS__);                     \
   } while (0)
-    LAUNCH_RUNS(decay_attention_runs_kernel, z, decays, query_start, state_slots, state, out, segment, segments, kept);
+#define LAUNCH_OWNED(VT)                                                                                                         \
+  do {                                                                                                                          \
+    if (is_float && activation) hipLaunchKernelGGL((decay_attention_runs_kernel<float, true, VT>), grid, dim3(64), 0, stream, (const float*)x, z, decays, query_start, state_slots, state, out, segment, segments, kept);   \
+    else if (is_float) hipLaunchKernelGGL((decay_attention_runs_kernel<float, false, VT>), grid, dim3(64), 0, stream, (const float*)x, z, decays, query_start, state_slots, state, out, segment, segments, kept);         \
+    else if (activation) hipLaunchKernelGGL((decay_attention_runs_kernel<bf16_t, true, VT>), grid, dim3(64), 0, stream, (const bf16_t*)x, z, decays, query_start, state_slots, state, out, segment, segments, kept);      \
+    else hipLaunchKernelGGL((decay_attention_runs_kernel<bf16_t, false, VT>), grid, dim3(64), 0, stream, (const bf16_t*)x, z, decays, query_start, state_slots, state, out, segment, segments, kept);                     \
+  } while (0)
+    if (owned == 4) LAUNCH_OWNED(most >= 4 ? 4 : 1);
+    else if (owned == 2) LAUNCH_OWNED(most >= 2 ? 2 : 1);
+    else LAUNCH_OWNED(1);
+#undef LAUNCH_OWNED
+    grid = dim3(vdim / 16, heads, requests * segments);
     if (segments > 1) {
       hipLaunchKernelGGL(decay_carry_kernel, dim3((D * vdim + 255) / 256, heads, requests), dim3(256), 0, stream, z, decays,
                          query_start, state_slots, state, segment, segments, carry);

@@ -97,6 +97,25 @@ def test_scale_heads_and_soft_cap(kernels, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,dim,vdim", [(16, 32, 128), (32, 16, 128), (40, 16, 64)])
+def test_decay_attention_of_many_heads(kernels, dtype, heads, dim, vdim):
+    """Enough (head, segment, columns) to go round the chip: a wave then owns two or four tiles of value columns."""
+    torch.manual_seed(heads)
+    counts = [300, 1, 530]
+    tokens, row = sum(counts), 2 * heads * dim + heads * vdim
+    decays = (1.0 - 2.0 ** -(1.0 + 8.0 * torch.rand(heads))).to(torch.float32)
+    state = 0.5 * torch.randn(4, heads, dim, vdim)
+    x = torch.randn(tokens, row).to(dtype)
+    batch = step_of(counts, [0] * 3, [2, 0, 3], "cuda")
+    plain_state, device_state = state.clone(), gpu(state)
+    want = TorchKernels(dtype).decay_attention(x, 0, heads * dim, 2 * heads * dim, heads, dim, vdim, decays, "silu", batch, plain_state)
+    got = kernels[dtype].decay_attention(gpu(x), 0, heads * dim, 2 * heads * dim, heads, dim, vdim, gpu(decays), "silu", batch, device_state)
+    scale = float(want.abs().max())
+    close(got / scale, want / scale, torch.float32, atol=2e-5, rtol=1e-4)
+    close(device_state, plain_state, torch.float32, atol=5e-5, rtol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("activation", ["silu", "sigmoid"])
 @pytest.mark.parametrize("heads,vdim", [(3, 40), (1, 300), (1, 1300)])
 def test_gated_head_norm_wide_and_squashed(kernels, dtype, activation, heads, vdim):
