@@ -32,7 +32,7 @@ class SozavikAttentionMixer:
     dim: int
     vdim: int
     scale: float
-    window: int
+    window: int | None
     v_mix: bool
     softcap: float | None = None
     rot: SozavikRotary | None = None
@@ -75,7 +75,9 @@ def _read_mixer(kind: str, values: dict[str, Any], where: str):
             raise ConfigError(f"{where}: 'decay' must list one number a head")
         return SozavikLightningMixer(heads=heads, dim=reader.integer("dim"), vdim=reader.integer("vdim"), decay=tuple(float(d) for d in decay))
     heads = reader.integer("heads")
-    mask = KeyReader(_mapping(values.get("mask"), f"{where}.mask"), f"{where}.mask")
+    window = None  # (no mask: every earlier token is seen)
+    if values.get("mask") is not None:
+        window = KeyReader(_mapping(values["mask"], f"{where}.mask"), f"{where}.mask").integer("size")
     rot, softcap = None, None
     if kind == "attention":
         found = KeyReader(_mapping(values.get("rot"), f"{where}.rot"), f"{where}.rot")
@@ -87,7 +89,7 @@ def _read_mixer(kind: str, values: dict[str, Any], where: str):
         softcap = reader.number("softcap") if reader.optional("softcap") is not None else None
     return SozavikAttentionMixer(
         heads=heads, kv_heads=reader.integer("kv_heads", default=heads), dim=reader.integer("dim"), vdim=reader.integer("vdim"),
-        scale=reader.number("scale"), window=mask.integer("size"), v_mix=reader.boolean("v_mix", default=False), softcap=softcap, rot=rot,
+        scale=reader.number("scale"), window=window, v_mix=reader.boolean("v_mix", default=False), softcap=softcap, rot=rot,
     )
 
 
@@ -168,7 +170,9 @@ class SozavikConfig(ArchitectureConfig):
                 described: dict[str, Any] = {"heads": mixer.heads, "dim": mixer.dim, "vdim": mixer.vdim, "decay": list(mixer.decay)}
             else:
                 described = {"heads": mixer.heads, "kv_heads": mixer.kv_heads, "dim": mixer.dim, "vdim": mixer.vdim,
-                             "scale": mixer.scale, "mask": {"size": mixer.window}, "v_mix": mixer.v_mix}
+                             "scale": mixer.scale, "v_mix": mixer.v_mix}
+                if mixer.window is not None:
+                    described["mask"] = {"size": mixer.window}
                 if mixer.rot is not None:
                     rot: dict[str, Any] = {"base": mixer.rot.base, "dims": mixer.rot.dims}
                     if mixer.rot.scaling is not None:

@@ -104,6 +104,11 @@ def window_attention(q, k, v, scale, window, cap=None, sinks=None):
     return out
 
 
+def window_of(m, n):
+    """The mask's size; a mixer without a mask sees every earlier token."""
+    return m["mask"]["size"] if m.get("mask") else n
+
+
 def mix_values(v, shared, tensors, prefix):
     """The first layer that mixes gives its values (a token's, all heads side by side) to the later ones: they take
     (1 - a) v + a v_first."""
@@ -128,7 +133,7 @@ def attention_mixer(h, positions, m, tensors, prefix, eps, shared):
     q, k = rotate_pairs(q, positions, frequencies), rotate_pairs(k, positions, frequencies)
     if m.get("v_mix"):
         v = mix_values(v, shared, tensors, prefix)
-    mixed = window_attention(q, k, v, m["scale"], m["mask"]["size"], cap=m["softcap"], sinks=tensors[prefix + "sink"])
+    mixed = window_attention(q, k, v, m["scale"], window_of(m, n), cap=m.get("softcap"), sinks=tensors[prefix + "sink"])
     gate = torch.sigmoid(h @ tensors[prefix + "g"].T)  # [n, H]
     mixed = mixed * gate[:, :, None]
     return mixed.reshape(n, H * dv) @ tensors[prefix + "o"].T
@@ -143,7 +148,7 @@ def attention_2_mixer(h, m, tensors, prefix, eps, shared):
     v = (h @ tensors[prefix + "v"].T).view(n, G, dv)
     if m.get("v_mix"):
         v = mix_values(v, shared, tensors, prefix)
-    mixed = window_attention(q.view(n, H, d), k.view(n, G, d), v, m["scale"], m["mask"]["size"])
+    mixed = window_attention(q.view(n, H, d), k.view(n, G, d), v, m["scale"], window_of(m, n))
     return mixed.reshape(n, H * dv) @ tensors[prefix + "o"].T
 
 

@@ -41,6 +41,10 @@ def test_config_round_trip_and_refusals():
     assert SozavikConfig.from_dict(config.to_config_json()) == config
     assert json.loads(json.dumps(config.to_config_json())) == cases.MIXED
     assert SozavikConfig.from_dict(cases.config_of([(cases.lightning(), None)], logit_softcap=None)).logit_softcap is None
+    unmasked = cases.config_of([(cases.attention_2(), None)])
+    del unmasked["layers"][0]["mixer"]["mask"]
+    assert SozavikConfig.from_dict(unmasked).layers[0].mixer.window is None
+    assert SozavikConfig.from_dict(SozavikConfig.from_dict(unmasked).to_config_json()) == SozavikConfig.from_dict(unmasked)
     broken = [
         cases.config_of([(cases.attention(heads=5, kv_heads=2), None)]),  # heads no multiple of kv_heads
         cases.config_of([(cases.attention(dims=26), None)]),  # more rotated dimensions than a head has
@@ -109,6 +113,9 @@ ALONE = {
         [(cases.attention(), cases.dense(8)), (cases.lightning(), None), (cases.attention_2(), None), (cases.attention(heads=4, kv_heads=4, dim=8, vdim=20, dims=4), None)]),
     "no layer mixes values": cases.config_of([(cases.attention(v_mix=False), None), (cases.attention_2(v_mix=False), None)]),
 }
+ALONE["no mask"] = cases.config_of([(cases.attention(), cases.dense(16)), (cases.attention_2(), None)])
+for _layer in ALONE["no mask"]["layers"]:
+    del _layer["mixer"]["mask"]
 
 
 @pytest.mark.parametrize("name", list(ALONE))
