@@ -28,7 +28,13 @@ __device__ __forceinline__ bf16x8 load8_stream(const bf16_t* p) { return *(const
 #define TARGET_WAVES 2048
 #endif
 
-template <int WAVES, int MT, typename TO, bool GATED>
+// GATED in the kernels for up to 64 rows below: 0 a plain product, 1 silu(gate) * up, 2 relu(gate) * up
+template <int GATED>
+__device__ __forceinline__ float gate_value(float gate) {
+  return GATED == 2 ? fmaxf(gate, 0.f) : gate / (1.f + expf(-gate));
+}
+
+template <int WAVES, int MT, typename TO, int GATED>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                                  const bf16_t* __restrict__ w,
                                                                  const void* __restrict__ bias, int bias_is_float,
@@ -132,7 +138,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
     for (int i = 0; i < 2; ++i) {
       if (n_first + 2 * i + 1 < N) {
         const float gate = total[2 * i], up = total[2 * i + 1];
-        dst[i] = from_float<TO>(gate / (1.f + expf(-gate)) * up);
+        dst[i] = from_float<TO>(gate_value<GATED>(gate) * up);
       }
     }
   } else {
@@ -143,7 +149,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
   }
 }
 
-template <int WAVES, int MT, typename TO, bool GATED>
+template <int WAVES, int MT, typename TO, int GATED>
 static int launch_skinny(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N,
                          int K, int splits, hipStream_t stream) {
   const size_t lds = (size_t)WAVES * MT * 64 * 4 * sizeof(float);
@@ -152,7 +158,7 @@ static int launch_skinny(const void* x, const void* w, const void* bias, int bia
   return LAUNCH_STATUS();
 }
 
-template <int WAVES, typename TO, bool GATED>
+template <int WAVES, typename TO, int GATED>
 static int pick_tiles(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N, int K,
                       int splits, hipStream_t stream) {
   if (M <= 16) return launch_skinny<WAVES, 1, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
@@ -160,7 +166,7 @@ static int pick_tiles(const void* x, const void* w, const void* bias, int bias_i
   return launch_skinny<WAVES, 4, TO, GATED>(x, w, bias, bias_is_float, out, M, N, K, splits, stream);
 }
 
-template <typename TO, bool GATED>
+template <typename TO, int GATED>
 static int pick_waves(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N, int K,
                       int splits, hipStream_t stream) {
   // enough waves to cover the chip (about 2,048), but no more than there are 128-wide groups of K
@@ -178,7 +184,7 @@ static int pick_waves(const void* x, const void* w, const void* bias, int bias_i
 // x doubles the traffic.  More tiles a wave also means more bytes under way a wave and fewer
 // workgroups: it pays for long K ranges and big weights (7B sizes at 8 rows: gate/up 57.7 -> 52.1 us
 // with two tiles, down 32.1 -> 26.3 us with four; 1.5B sizes at 16 rows: gate/up 18.0 -> 16.9 us).
-template <int WAVES, int NT, typename TO, bool GATED>
+template <int WAVES, int NT, typename TO, int GATED>
 __global__ __launch_bounds__(WAVES * 64) void gemm_pair_kernel(const bf16_t* __restrict__ x,
                                                                const bf16_t* __restrict__ w,
                                                                const void* __restrict__ bias, int bias_is_float,
@@ -254,7 +260,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_pair_kernel(const bf16_t* __r
     for (int i = 0; i < 2; ++i) {
       if (n_first + 2 * i + 1 < N) {
         const float gate = total[2 * i], up = total[2 * i + 1];
-        dst[i] = from_float<TO>(gate / (1.f + expf(-gate)) * up);
+        dst[i] = from_float<TO>(gate_value<GATED>(gate) * up);
       }
     }
   } else {
@@ -265,7 +271,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_pair_kernel(const bf16_t* __r
   }
 }
 
-template <int NT, typename TO, bool GATED>
+template <int NT, typename TO, int GATED>
 static int launch_pair(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N,
                        int K, int splits, hipStream_t stream) {
   const size_t lds = (size_t)4 * NT * 64 * 4 * sizeof(float);
@@ -313,7 +319,7 @@ __device__ __forceinline__ void stream_wait_loads() {
 
 // MT: 16-row tiles of x (up to 16 MT rows).  A stage then holds MT chunks of x beside the NT of the
 // weights for every step, and each weight operand meets MT operands of x.
-template <int WAVES, int NT, int MT, int G, typename TO, bool GATED>
+template <int WAVES, int NT, int MT, int G, typename TO, int GATED>
 __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(const bf16_t* __restrict__ x,
                                                                  const bf16_t* __restrict__ w,
                                                                  const void* __restrict__ bias, int bias_is_float,
@@ -427,7 +433,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(const bf16_t* _
       for (int i = 0; i < 2; ++i) {
         if (n_first + 2 * i + 1 < N) {
           const float gate = total[2 * i], up = total[2 * i + 1];
-          dst[i] = from_float<TO>(gate / (1.f + expf(-gate)) * up);
+          dst[i] = from_float<TO>(gate_value<GATED>(gate) * up);
         }
       }
     } else {
@@ -439,7 +445,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(const bf16_t* _
   }
 }
 
-template <int WAVES, int NT, int MT, int G, typename TO, bool GATED>
+template <int WAVES, int NT, int MT, int G, typename TO, int GATED>
 static int launch_stream(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N,
                          int K, int splits, hipStream_t stream) {
   const size_t stages = (size_t)WAVES * STREAM_STAGES * (NT + MT) * G * STREAM_CHUNK;
@@ -467,7 +473,7 @@ static int launch_stream(const void* x, const void* w, const void* bias, int bia
 // for four tiles that share its x (the down projections and the 32B sizes' gate/up) gemm_pair's
 // registers stay ahead, and the caller keeps it there.
 // M <= 16, K / splits a multiple of 128.
-template <typename TO, bool GATED>
+template <typename TO, int GATED>
 static int pick_stream(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int M, int N, int K,
                        int splits, hipStream_t stream, int nt = 0, int g = 0) {
   const long tiles = (N + 15) / 16;
@@ -503,7 +509,7 @@ static int pick_stream(const void* x, const void* w, const void* bias, int bias_
 static int stream_entry(const void* x, const void* w, const void* bias, int bias_is_float, void* out, int out_is_float,
                         int gated, int M, int N, int K, int splits, hipStream_t stream, int nt, int g) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || K <= 0 || splits < 1 || K % splits || (K / splits) % (STEP * GROUP) || (gated && N % 2))
+  if (M > 64 || K <= 0 || splits < 1 || K % splits || (K / splits) % (STEP * GROUP) || (gated && N % 2) || gated > 1)
     return ERR_BAD_ARGUMENT;
   if (splits > 1 && (gated || !out_is_float)) return ERR_BAD_ARGUMENT;
   if (gated)
@@ -808,7 +814,7 @@ extern "C" int llmserve_gemm_medium(const void* x, const void* w, const void* bi
                                     int out_is_float, int gated, int M, int N, int K, int splits,
                                     hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || K <= 0 || K % (STEP * GROUP) || (gated && N % 2) || splits < 1) return ERR_BAD_ARGUMENT;
+  if (M > 64 || K <= 0 || K % (STEP * GROUP) || (gated && N % 2) || splits < 1 || gated > 1) return ERR_BAD_ARGUMENT;  // (these epilogues know silu alone)
   if (splits > 1 && (gated || !out_is_float)) return ERR_BAD_ARGUMENT;
   if (gated)
     return out_is_float ? pick_medium<float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)
@@ -1088,7 +1094,7 @@ extern "C" int llmserve_gemm_ring(const void* x, const void* w, const void* bias
                                   int out_is_float, int gated, int M, int N, int K, int splits, int nt,
                                   hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 128 || K <= 0 || splits < 1 || K % splits || (gated && N % 2)) return ERR_BAD_ARGUMENT;
+  if (M > 128 || K <= 0 || splits < 1 || K % splits || (gated && N % 2) || gated > 1) return ERR_BAD_ARGUMENT;  // (these epilogues know silu alone)
   if (splits > 1 && (gated || !out_is_float)) return ERR_BAD_ARGUMENT;
   if (gated)
     return out_is_float ? pick_ring<float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream, nt)
@@ -1525,7 +1531,7 @@ static int pick_tiled(const void* x, const void* w, const void* bias, int bias_i
 extern "C" int llmserve_gemm_tiled(const void* x, const void* w, const void* bias, int bias_is_float, void* out,
                                    int out_is_float, int gated, int M, int N, int K, int splits, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || K % TILE_K || (gated && N % 2) || splits < 1) return ERR_BAD_ARGUMENT;
+  if (K <= 0 || K % TILE_K || (gated && N % 2) || splits < 1 || gated > 1) return ERR_BAD_ARGUMENT;  // (these epilogues know silu alone)
   if (splits > 1 && (gated || !out_is_float || K % splits || (K / splits) % TILE_K)) return ERR_BAD_ARGUMENT;
   if (gated)
     return out_is_float ? pick_tiled<float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)
@@ -1535,14 +1541,14 @@ extern "C" int llmserve_gemm_tiled(const void* x, const void* w, const void* bia
 }
 
 // x, w bfloat16; out bfloat16 or float32.  Needs 1 <= M <= 64, K a multiple of 32, and with
-// `gated` an even N.  Any N.  With splits > 1 (float32 out, not gated, K / splits a multiple of
+// `gated` (1: silu(gate) * up, 2: relu(gate) * up) an even N.  Any N.  With splits > 1 (float32 out, not gated, K / splits a multiple of
 // 32) `out` is [splits, M, N]: slice s holds the sums over the s-th part of K (the bias in slice 0),
 // and whoever reads it adds the slices in order.
 extern "C" int llmserve_gemm_skinny(const void* x, const void* w, const void* bias, int bias_is_float, void* out,
                                     int out_is_float, int gated, int M, int N, int K, int splits,
                                     hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || K <= 0 || K % STEP || (gated && N % 2) || splits < 1) return ERR_BAD_ARGUMENT;
+  if (M > 64 || K <= 0 || K % STEP || (gated && N % 2) || gated > 2 || splits < 1) return ERR_BAD_ARGUMENT;
   if (splits > 1 && (gated || !out_is_float || K % splits || (K / splits) % STEP)) return ERR_BAD_ARGUMENT;
   if (M <= 16 && (K / splits) % (STEP * GROUP) == 0) {
     // several weight tiles a wave where a wave has many groups of K to walk (or x is all 16 rows) and
@@ -1555,6 +1561,9 @@ extern "C" int llmserve_gemm_skinny(const void* x, const void* w, const void* bi
                                                                                                             : 1;
     // Two tiles or one: through LDS (gemm_stream), unless many rows of x meet a long walk over K.
     if (share != 4 && !(share == 2 && M > 8 && per_wave >= 4)) {
+      if (gated == 2)
+        return out_is_float ? pick_stream<float, 2>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)
+                            : pick_stream<bf16_t, 2>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
       if (gated)
         return out_is_float ? pick_stream<float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)
                             : pick_stream<bf16_t, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
@@ -1563,6 +1572,9 @@ extern "C" int llmserve_gemm_skinny(const void* x, const void* w, const void* bi
     }
 #define PAIR_CASE(NT)                                                                                              \
   if (share == NT) {                                                                                               \
+    if (gated == 2)                                                                                                \
+      return out_is_float ? launch_pair<NT, float, 2>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)          \
+                          : launch_pair<NT, bf16_t, 2>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);        \
     if (gated)                                                                                                     \
       return out_is_float ? launch_pair<NT, float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)       \
                           : launch_pair<NT, bf16_t, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);     \
@@ -1584,6 +1596,9 @@ extern "C" int llmserve_gemm_skinny(const void* x, const void* w, const void* bi
     return out_is_float ? pick_stream<float, false>(x, w, bias, bias_is_float, out, M, N, K, splits, stream, 1, g)
                         : pick_stream<bf16_t, false>(x, w, bias, bias_is_float, out, M, N, K, 1, stream, 1, g);
   }
+  if (gated == 2)
+    return out_is_float ? pick_waves<float, 2>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)
+                        : pick_waves<bf16_t, 2>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);
   if (gated)
     return out_is_float ? pick_waves<float, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream)
                         : pick_waves<bf16_t, true>(x, w, bias, bias_is_float, out, M, N, K, 1, stream);

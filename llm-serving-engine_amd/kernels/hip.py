@@ -333,8 +333,9 @@ class HipKernels:
         return LinearWeights(weight, bias)
 
     def prepare_gated_linear(self, gate: torch.Tensor, up: torch.Tensor, activation: str = "silu") -> GatedLinearWeights:
-        """`activation` is the gate's: silu is applied in the epilogue of the product itself; the others
-        (gelu, gelu_tanh, relu) by a kernel of their own behind a plain product."""
+        """`activation` is the gate's: silu is applied in the epilogue of the product itself, relu too where the
+        product has few rows; the others (gelu, gelu_tanh, and relu over many rows) by a kernel of their own
+        behind a plain product."""
         if activation not in _ACTIVATIONS:
             raise KernelError(f"gated_linear: no kernel applies the activation {activation!r} (known: {', '.join(_ACTIVATIONS)})")
         if gate.shape != up.shape:
@@ -642,6 +643,18 @@ class HipKernels:
     def gated_linear(self, x: torch.Tensor, weights: GatedLinearWeights) -> torch.Tensor:
         """silu (or another activation) of the even rows' products times the odd rows'."""
         out = self._empty((x.shape[0], weights.width), self.dtype)
+        if (
+            weights.activation == "relu"
+            and self.dtype == torch.bfloat16
+            and self._streaming(x, weights.both, gated=True) == "skinny"
+        ):
+            # the kernels for a few rows (a decode step) apply relu in their epilogue too: one launch less a layer
+            status = self._gemm_bf16.llmserve_gemm_skinny(
+                _pointer(x), _pointer(weights.both.weight), _pointer(None), 0, _pointer(out), _is_float(out), 2,
+                x.shape[0], 2 * weights.width, x.shape[1], 1, self._stream,
+            )
+            _check(status, "gated_linear")
+            return out
         if weights.activation != "silu":  # no fused epilogue: the product plain, the activation behind it
             both = self.linear(x, weights.both, out_dtype=torch.bfloat16 if self._library(x, weights.both) else torch.float32)
             status = self._elementwise.llmserve_gate_mul(

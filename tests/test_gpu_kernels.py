@@ -874,10 +874,11 @@ def test_rotation_store_and_attention_of_prompt_portions(kernels, dtype, pairing
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("activation", ["silu", "gelu", "gelu_tanh", "relu"])
-@pytest.mark.parametrize("rows,inner,outer", [(5, 96, 200), (70, 64, 333), (300, 128, 1000)])
+@pytest.mark.parametrize("rows,inner,outer", [(5, 96, 200), (16, 512, 520), (40, 128, 264), (70, 64, 333), (300, 128, 1000)])
 def test_gated_products_with_every_gate_activation(kernels, dtype, activation, rows, inner, outer):
-    """The gate's activation is a parameter of the gated product: SiLU is applied in the products' own epilogues,
-    the others by the activation kernel behind a plain product; one that has no kernel is refused by name."""
+    """The gate's activation is a parameter of the gated product: SiLU is applied in the products' own epilogues (relu
+    too in those for a few rows), the others by the activation kernel behind a plain product; one that has no kernel
+    is refused by name."""
     k = kernels[dtype]
     acts = {"silu": F.silu, "gelu": F.gelu, "gelu_tanh": lambda z: F.gelu(z, approximate="tanh"), "relu": torch.relu}
     x, gate, up = torch.randn(rows, inner), torch.randn(outer, inner) / math.sqrt(inner), torch.randn(outer, inner) / math.sqrt(inner)
