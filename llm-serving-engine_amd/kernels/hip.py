@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import contextlib
 import ctypes
+import types
 from dataclasses import dataclass
 from typing import Any
 
@@ -1378,9 +1379,8 @@ class HipKernels:
         )
         _check(status, "assemble_heads")
         if store and not here:
-            from ..parts.position import HeadLayout
-
-            self.rotate_and_store(out, HeadLayout(heads, kv_heads, width), batch, cell, None, "none")
+            layout = types.SimpleNamespace(num_heads=heads, num_kv_heads=kv_heads, head_dim=width, width=(heads + 2 * kv_heads) * width)
+            self.rotate_and_store(out, layout, batch, cell, None, "none")
         return out
 
     def scale_heads(self, x, heads: int, width: int, gates, gate_first: int, squash: str) -> torch.Tensor:
